@@ -281,6 +281,201 @@ def architecture_name(d: Dict[str, Any], where: str = "config.json") -> str:
     """``architectures[0]``, the key the reference selects the model class by
     (minivllm/models/loader.py:10)."""
     archs = d.get("architectures")
+    if archs is None and isinstance(d.get("architecture"), str):
+        return d["architecture"]             # configurations that name their one architecture directly
     if not isinstance(archs, (list, tuple)) or not archs or not isinstance(archs[0], str):
         raise ConfigError(f"{where}: 'architectures' must be a non-empty list of names")
     return archs[0]
+
+
+# ---------------------------------------------------------------------------------------
+# Bolapel
+# ---------------------------------------------------------------------------------------
+def _section(d: Dict[str, Any], key: str, where: str, optional: bool = False) -> Optional[Dict[str, Any]]:
+    v = d.get(key)
+    if v is None:
+        if optional:
+            return None
+        raise ConfigError(f"{where}: required section '{key}' is missing")
+    if not isinstance(v, dict):
+        raise ConfigError(f"{where}: '{key}' must be an object, got {v!r}")
+    return v
+
+
+@dataclass(frozen=True)
+class BolapelLayer:
+    """One entry of Bolapel's ``layers``. ``type`` is "general_delta" (heads, dim) or "attention"
+    (heads, kv_heads, dim, vdim, scale, the chunk of its mask, the rotation's dims and base, and
+    ``kv_from``: the layer whose keys and values it reads instead of making its own). ``ff`` is the
+    width of the layer's dense feed-forward, None for a layer without one."""
+    type: str
+    heads: int
+    dim: int
+    kv_heads: int = 0
+    vdim: int = 0
+    scale: float = 1.0
+    chunk: Optional[int] = None
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    kv_from: Optional[int] = None
+    ff: Optional[int] = None
+    # general_delta: rows of the first of the two small matrices behind the decay. config.json need not
+    # state it (key "rank"); the stored tensor's shape does, and the loader fills it in from there
+    decay_rank: Optional[int] = None
+
+    def mixer_dict(self) -> Dict[str, Any]:
+        if self.type == "general_delta":
+            m = {"heads": self.heads, "dim": self.dim}
+            if self.decay_rank is not None:
+                m["rank"] = self.decay_rank
+            return m
+        m: Dict[str, Any] = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim,
+                             "scale": self.scale}
+        if self.chunk is not None:
+            m["mask"] = {"size": self.chunk}
+        if self.rot_dims:
+            m["rot"] = {"dims": self.rot_dims, "base": self.rot_base}
+        if self.kv_from is not None:
+            m["kv_from"] = self.kv_from
+        return m
+
+
+@dataclass(frozen=True)
+class BolapelConfig(ModelConfig):
+    """Bolapel: a decoder whose layers are listed one by one in ``layers``; each has a mixer (a
+    generalised delta rule with a matrix state per head, or sigmoid-weighted attention inside chunks
+    of the sequence, possibly on another layer's keys and values) and optionally a dense gated
+    feed-forward, every sublayer with a norm in front and behind and a token shift in front of the
+    mixer. Keys: ``vocab``, ``width``, ``layers``, ``norm.eps``, ``logit_softcap``; the architecture
+    is named by ``architecture``. The model states no longest sequence; ``max_position_embeddings``
+    here only bounds what an engine may be asked to serve."""
+
+    architecture: ClassVar[str] = "Bolapel"
+
+    vocab_size: int = 0
+    hidden_size: int = 0
+    layers: Tuple[BolapelLayer, ...] = ()
+    norm_eps: float = 1e-5
+    logit_softcap: Optional[float] = None
+    max_position_embeddings: int = 1 << 24
+    dtype: str = "bfloat16"
+    eos_token_ids: Tuple[int, ...] = ()
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any], where: str = "config.json") -> "BolapelConfig":
+        raw_layers = d.get("layers")
+        if not isinstance(raw_layers, (list, tuple)) or not raw_layers:
+            raise ConfigError(f"{where}: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(raw_layers):
+            lw = f"{where}: layers[{i}]"
+            if not isinstance(entry, dict):
+                raise ConfigError(f"{lw} must be an object")
+            kind = entry.get("type")
+            m = _section(entry, "mixer", lw)
+            mw = lw + ".mixer"
+            mlp = _section(entry, "mlp", lw, optional=True)
+            ff = None
+            if mlp is not None:
+                if mlp.get("kind", "dense") != "dense":
+                    raise ConfigError(f"{lw}.mlp: kind {mlp.get('kind')!r} is not supported (dense only)")
+                ff = _require(mlp, "ff", int, lw + ".mlp")
+            if kind == "general_delta":
+                rank = m.get("rank")
+                layers.append(BolapelLayer(type=kind, heads=_require(m, "heads", int, mw),
+                                           dim=_require(m, "dim", int, mw), ff=ff,
+                                           decay_rank=None if rank is None else _typed(rank, "rank", int, mw)))
+            elif kind == "attention":
+                mask = _section(m, "mask", mw, optional=True)
+                rot = _section(m, "rot", mw, optional=True)
+                heads = _require(m, "heads", int, mw)
+                dim = _require(m, "dim", int, mw)
+                kv_heads = m.get("kv_heads")
+                vdim = m.get("vdim")
+                kv_from = m.get("kv_from")
+                layers.append(BolapelLayer(
+                    type=kind, heads=heads, dim=dim,
+                    kv_heads=heads if kv_heads is None else _typed(kv_heads, "kv_heads", int, mw),
+                    vdim=dim if vdim is None else _typed(vdim, "vdim", int, mw),
+                    scale=_require(m, "scale", float, mw),
+                    chunk=None if mask is None else _require(mask, "size", int, mw + ".mask"),
+                    rot_dims=0 if rot is None else _require(rot, "dims", int, mw + ".rot"),
+                    rot_base=10000.0 if rot is None else _require(rot, "base", float, mw + ".rot"),
+                    kv_from=None if kv_from is None else _typed(kv_from, "kv_from", int, mw), ff=ff))
+            else:
+                raise ConfigError(f"{lw}: layer type {kind!r} is not supported (general_delta, attention)")
+        norm = _section(d, "norm", where)
+        cap = d.get("logit_softcap")
+        dtype = d.get("dtype", d.get("torch_dtype", "bfloat16")) or "bfloat16"
+        if str(dtype) not in _DTYPE_NAMES:
+            raise ConfigError(f"{where}: unknown dtype {dtype!r}")
+        eos = d.get("eos_token_id")
+        eos_ids: Tuple[int, ...] = ()
+        if isinstance(eos, int) and not isinstance(eos, bool):
+            eos_ids = (eos,)
+        elif isinstance(eos, (list, tuple)) and all(isinstance(e, int) for e in eos):
+            eos_ids = tuple(eos)
+        elif eos is not None:
+            raise ConfigError(f"{where}: eos_token_id must be an integer or a list of integers, got {eos!r}")
+        max_pos = d.get("max_position_embeddings")
+        cfg = cls(
+            vocab_size=_require(d, "vocab", int, where),
+            hidden_size=_require(d, "width", int, where),
+            layers=tuple(layers),
+            norm_eps=_require(norm, "eps", float, where + ".norm"),
+            logit_softcap=None if cap is None else _typed(cap, "logit_softcap", float, where),
+            max_position_embeddings=(1 << 24) if max_pos is None else _typed(max_pos, "max_position_embeddings", int, where),
+            dtype=_DTYPE_NAMES[str(dtype)],
+            eos_token_ids=eos_ids,
+        )
+        cfg.validate(where)
+        return cfg
+
+    def validate(self, where: str = "config") -> None:
+        if self.vocab_size <= 0 or self.hidden_size <= 0:
+            raise ConfigError(f"{where}: vocab and width must be positive")
+        if self.norm_eps <= 0:
+            raise ConfigError(f"{where}: norm.eps must be positive, got {self.norm_eps}")
+        if self.logit_softcap is not None and self.logit_softcap <= 0:
+            raise ConfigError(f"{where}: logit_softcap must be positive, got {self.logit_softcap}")
+        for i, l in enumerate(self.layers):
+            lw = f"{where}: layers[{i}]"
+            if l.heads <= 0 or l.dim <= 0:
+                raise ConfigError(f"{lw}: heads and dim must be positive")
+            if l.ff is not None and l.ff <= 0:
+                raise ConfigError(f"{lw}: mlp.ff must be positive")
+            if l.type != "attention":
+                continue
+            if l.kv_heads <= 0 or l.vdim <= 0 or l.heads % l.kv_heads:
+                raise ConfigError(f"{lw}: {l.heads} heads are not a multiple of {l.kv_heads} kv_heads (or vdim <= 0)")
+            if l.chunk is not None and l.chunk < 1:
+                raise ConfigError(f"{lw}: mask.size must be >= 1, got {l.chunk}")
+            if l.rot_dims < 0 or l.rot_dims % 2 or l.rot_dims > l.dim:
+                raise ConfigError(f"{lw}: rot.dims {l.rot_dims} must be even and at most dim {l.dim}")
+            if l.rot_dims and l.rot_base <= 0:
+                raise ConfigError(f"{lw}: rot.base must be positive")
+            if l.kv_from is not None:
+                j = l.kv_from
+                if not (0 <= j < i) or self.layers[j].type != "attention" or self.layers[j].kv_from is not None:
+                    raise ConfigError(f"{lw}: kv_from {j} must name an earlier attention layer with keys of its own")
+                o = self.layers[j]
+                if (o.kv_heads, o.dim, o.vdim, o.rot_dims, o.rot_base) != (l.kv_heads, l.dim, l.vdim, l.rot_dims, l.rot_base):
+                    raise ConfigError(f"{lw}: kv_from {j} has other key/value heads, sizes or rotation than this layer")
+
+    def to_dict(self) -> Dict[str, Any]:
+        d: Dict[str, Any] = {
+            "architecture": self.architecture,
+            "layers": [{"type": l.type, "mixer": l.mixer_dict(),
+                        "mlp": None if l.ff is None else {"kind": "dense", "ff": l.ff}} for l in self.layers],
+            "norm": {"eps": self.norm_eps},
+            "vocab": self.vocab_size,
+            "width": self.hidden_size,
+            "torch_dtype": self.dtype,
+        }
+        if self.logit_softcap is not None:
+            d["logit_softcap"] = self.logit_softcap
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids) if len(self.eos_token_ids) > 1 else self.eos_token_ids[0]
+        if self.max_position_embeddings != (1 << 24):
+            d["max_position_embeddings"] = self.max_position_embeddings
+        return d

@@ -889,3 +889,76 @@ extern "C" int mv_swiglu(const void* gate_up, void* out, int n, int I, int dtype
                                      (T*)out, total, I));
     return mv_check_launch("swiglu");
 }
+
+// ---------------------------------------------------------------------------------------
+// A norm behind a sublayer, the residual add, and the norm in front of the next sublayer:
+//   v = resid[r] + y[r] / sqrt(mean(y[r]^2) + eps_a) * wa ;  resid[r] = v ;
+//   out[r] = v / sqrt(mean(v^2) + eps_b) * wb                          (out == null: the add alone)
+// One workgroup per row; the sum stays float from the first norm to the second.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_a, int unit_a, float* __restrict__ resid,
+                     WeightPtr wb, float eps_b, int unit_b, T* __restrict__ out, int h) {
+    __shared__ float scratch[17];
+    const int r = blockIdx.x;
+    const T* yr = y + (size_t)r * ldy;
+    float* x = resid + (size_t)r * h;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < h; c += blockDim.x) {
+        const float v = to_f(yr[c]);
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, scratch);
+    const float ra = 1.f / sqrtf(ss / (float)h + eps_a);
+    float ss2 = 0.f;
+    for (int c = threadIdx.x; c < h; c += blockDim.x) {
+        float w = wa.at(c);
+        if (unit_a) w += 1.f;
+        const float v = x[c] + to_f(yr[c]) * ra * w;
+        x[c] = v;
+        ss2 = fmaf(v, v, ss2);
+    }
+    if (out == nullptr) return;
+    ss2 = block_sum(ss2, scratch);
+    const float rb = 1.f / sqrtf(ss2 / (float)h + eps_b);
+    T* o = out + (size_t)r * h;
+    for (int c = threadIdx.x; c < h; c += blockDim.x) {
+        float w = wb.at(c);
+        if (unit_b) w += 1.f;
+        o[c] = from_f<T>(x[c] * rb * w);      // the thread's own store of x[c] above
+    }
+}
+
+extern "C" int mv_norm_add_norm(const void* y, long ldy, const void* wa, int wa_dtype, float eps_a, int unit_a,
+                                float* resid, const void* wb, int wb_dtype, float eps_b, int unit_b, void* out, int n,
+                                int h, int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && h > 0 && ldy >= h, "norm_add_norm: bad sizes n=%d h=%d", n, h);
+    MV_REQUIRE(y && wa && resid && mv_valid_dtype(wa_dtype) && eps_a > 0.f, "norm_add_norm: missing operand");
+    MV_REQUIRE(out == nullptr || (wb && mv_valid_dtype(wb_dtype) && eps_b > 0.f), "norm_add_norm: the second norm lacks its weight");
+    if (n == 0) return 0;
+    WeightPtr pa{wa, wa_dtype}, pb{wb, out ? wb_dtype : MV_F32};
+    MV_DISPATCH_T(dtype, "norm_add_norm",
+                  hipLaunchKernelGGL(norm_add_norm_kernel<T>, dim3(n), dim3(256), 0, stream, (const T*)y, ldy, pa, eps_a,
+                                     unit_a, resid, pb, eps_b, unit_b, (T*)out, h));
+    return mv_check_launch("norm_add_norm");
+}
+
+// ---------------------------------------------------------------------------------------
+// Soft cap of float logits, in place: x <- cap * tanh(x / cap).
+// ---------------------------------------------------------------------------------------
+__global__ void soft_cap_kernel(float* __restrict__ x, long ld, int cols, long total, float cap) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    float* p = x + (i / cols) * ld + (i % cols);
+    *p = cap * tanhf(*p / cap);
+}
+
+extern "C" int mv_soft_cap(float* x, long ld, int rows, int cols, float cap, hipStream_t stream) {
+    MV_REQUIRE(rows >= 0 && cols > 0 && ld >= cols && cap > 0.f, "soft_cap: bad sizes rows=%d cols=%d cap=%f", rows, cols,
+               (double)cap);
+    const long total = (long)rows * cols;
+    if (total == 0) return 0;
+    hipLaunchKernelGGL(soft_cap_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, x, ld, cols, total, cap);
+    return mv_check_launch("soft_cap");
+}

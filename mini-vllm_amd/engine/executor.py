@@ -109,6 +109,8 @@ class Executor:
         else:
             arch, model_config, source = model
             where = "the given tensors"
+        if arch.complete is not None:
+            model_config = arch.complete(model_config, source)
         self.arch, self.model_config = arch, model_config
         self.dtype = dtype_from_name(compute_dtype_name(config.dtype, getattr(model_config, "dtype", None), where))
         self.page_size = config.kv_cache_block_size
@@ -167,7 +169,7 @@ class Executor:
         self._next_token_buffer = 0
         self.kv_pages: Dict[int, Dict[str, torch.Tensor]] = {}     # per call with a cache need: its page tensors by name
         self._poison: Dict[int, List[int]] = {}                    # debug_poison_pages: pages to fill, per group
-        self.state_tensors: Dict[int, torch.Tensor] = {}
+        self.state_tensors: Dict[int, Dict[str, torch.Tensor]] = {}   # per call with state: its tensors by name
         self.num_pages = 0                                         # of the largest pool
         self.group_pages: List[int] = [0] * len(self.groups)       # pages of each group's pool
         self._allocate_memory()
@@ -212,11 +214,11 @@ class Executor:
 
     def _allocate_memory(self) -> None:
         cfg = self.config
-        for call, shape in enumerate(self.state_shapes):
-            if shape is not None:
-                dims, dt = shape
-                self.state_tensors[call] = torch.zeros((self.num_state_slots,) + tuple(dims), dtype=dt,
-                                                       device=self.device)
+        for call, shapes in enumerate(self.state_shapes):
+            if shapes is not None:
+                self.state_tensors[call] = {name: torch.zeros((self.num_state_slots,) + tuple(dims), dtype=dt,
+                                                              device=self.device)
+                                            for name, (dims, dt) in shapes.items()}
         if cfg.kv_cache_num_blocks is not None:
             given = cfg.kv_cache_num_blocks
             sizes = [int(given)] * len(self.groups) if isinstance(given, int) else [int(n) for n in given]
@@ -510,8 +512,9 @@ class Executor:
         fresh = [s.state_slot for s in seqs if s.start == 0]
         if fresh:
             index = torch.tensor(fresh, dtype=torch.int64, device=self.device)
-            for t in self.state_tensors.values():
-                t.index_fill_(0, index, 0)
+            for tensors in self.state_tensors.values():
+                for t in tensors.values():
+                    t.index_fill_(0, index, 0)
 
     def _context_cap(self, seqs: Sequence[SeqStep]) -> int:
         """The context length a decode graph is planned for: the next power of two (at least
@@ -664,7 +667,7 @@ class Executor:
         try:
             self.rt.workspace = self._graph_workspace
             meta = torch.empty(arr.size, dtype=torch.int32, device=self.device)
-            self._upload(arr, dst=meta)
+            self._upload(self._inert(arr, off), dst=meta)
             ctx = self._context(meta, off, facts, seqs)
             ctx.attention_plan.max_context_len = cap
             o = off["extra"][0]
@@ -820,6 +823,17 @@ class Executor:
         logger.info("recorded %d decode graphs ahead of serving", made)
         return made
 
+    def _inert(self, arr: np.ndarray, off) -> np.ndarray:
+        """What the runs that prepare a recording take as their step: the step itself, or, for a model
+        whose requests carry state from step to step, a copy with every row a padding row. Such a
+        run would otherwise advance the state a second time (writing the same keys twice is harmless);
+        the caller uploads the real step before it replays the graph."""
+        if not self.has_state:
+            return arr
+        inert = arr.copy()
+        self._as_padding(inert, off)
+        return inert
+
     @staticmethod
     def _as_padding(arr: np.ndarray, off) -> None:
         """Turns the rows of a packed step into padding rows: every kernel runs, none touches the cache."""
@@ -844,7 +858,7 @@ class Executor:
             self._prepare_graph_workspace()
             self.rt.workspace = self._graph_workspace
             meta = torch.empty(arr.size, dtype=torch.int32, device=self.device)
-            self._upload(arr, dst=meta)
+            self._upload(self._inert(arr, off), dst=meta)
             ctx = self._context(meta, off, facts, seqs)
             # the graph serves every context length up to its cap
             plan = ctx.attention_plan

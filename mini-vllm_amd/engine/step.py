@@ -118,7 +118,7 @@ class StepContext:
         self.attention_plan: Optional[AttentionPlan] = None
         # filled by the executor
         self._kv: Dict[int, "KVView"] = {}
-        self._state: Dict[int, torch.Tensor] = {}
+        self._state: Dict[int, Dict[str, torch.Tensor]] = {}
         self.page_size = 0
         # rows that a position encoding had gathered for this step (PositionEncoding.step_gather), by part
         self.position_rows: Dict[object, torch.Tensor] = {}
@@ -129,8 +129,10 @@ class StepContext:
         except KeyError:
             raise KeyError(f"call {call} has no cache: its mixer declared no cache need") from None
 
-    def state(self, call: int) -> torch.Tensor:
+    def state(self, call: int, name: str = "state") -> torch.Tensor:
+        """``[slots, *shape]`` of the state ``name`` of a call ("state": the one a mixer's
+        ``state_shape`` declares)."""
         try:
-            return self._state[call]
+            return self._state[call][name]
         except KeyError:
-            raise KeyError(f"call {call} has no state: its mixer declared no state shape") from None
+            raise KeyError(f"call {call} has no state {name!r}: neither its mixer nor its block declared it") from None

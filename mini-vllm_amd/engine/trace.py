@@ -37,7 +37,7 @@ class TraceError(RuntimeError):
 
 class TraceRunner:
     def __init__(self, model: str, dtype: str, max_tokens: int, page_size: int = 16, use_graph: bool = True,
-                 max_live: int = 16, enable_prefix_caching: bool = False, poison_pages: bool = False):
+                 max_live: int = 4, enable_prefix_caching: bool = False, poison_pages: bool = False):
         if TOKEN_ROUNDING % page_size:
             raise ValueError(f"the page size {page_size} must divide {TOKEN_ROUNDING}")
         max_tokens = max(TOKEN_ROUNDING, -(-max_tokens // TOKEN_ROUNDING) * TOKEN_ROUNDING)
@@ -105,10 +105,10 @@ class TraceRunner:
 
 
 def run(model: str, dtype: str, out_dir: str, max_tokens: int, stdin: IO[str], stdout: IO[str],
-        page_size: int = 16, use_graph: bool = True, enable_prefix_caching: bool = False) -> int:
+        page_size: int = 16, use_graph: bool = True, enable_prefix_caching: bool = False, max_live: int = 4) -> int:
     os.makedirs(out_dir, exist_ok=True)
     runner = TraceRunner(model, dtype, max_tokens, page_size=page_size, use_graph=use_graph,
-                         enable_prefix_caching=enable_prefix_caching)
+                         enable_prefix_caching=enable_prefix_caching, max_live=max_live)
     for line in stdin:
         line = line.strip()
         if not line:

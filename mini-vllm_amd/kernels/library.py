@@ -45,6 +45,28 @@ _SIGNATURES = {
                             c_int, c_int, c_int, c_void_p]),
     "mv_attention_ref": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                  c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
+    # h, ldh, out, ldo, mix, mix_dtype, state, token_seq, cu_seqlens, state_slots, n, width, dtype, stream
+    "mv_token_shift": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_int, c_int, c_int, c_void_p]),
+    # packed, ld, n, H, D, rank, w2, w0, a_bias, weight_dtype, decay_rate, key_eps, token_seq, coef, dtype, stream
+    "mv_delta_prepare": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                 c_float, c_float, c_void_p, c_void_p, c_int, c_void_p]),
+    # packed, ld, coef, state, cu_seqlens, state_slots, n_seqs, n, H, D, out, dtype, stream
+    "mv_delta_scan": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                              c_void_p, c_int, c_void_p]),
+    # raw, packed, ld, weight, weight_dtype, n, H, D, eps, out, ldo, dtype, stream
+    "mv_delta_finish": (c_int, [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p,
+                                c_long, c_int, c_void_p]),
+    # q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width, page_size, positions, token_seq,
+    # n, H, Hkv, D, Dv, scale, chunk, window, bias, gate, gate_stride, dtype, stream
+    "mv_attention_sigmoid_ref": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                         c_void_p, c_void_p, c_long, c_int, c_void_p]),
+    # y, ldy, wa, wa_dtype, eps_a, unit_a, resid, wb, wb_dtype, eps_b, unit_b, out, n, h, dtype, stream
+    "mv_norm_add_norm": (c_int, [c_void_p, c_long, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p, c_int, c_float,
+                                 c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
+    # x, ld, rows, cols, cap, stream
+    "mv_soft_cap": (c_int, [c_void_p, c_long, c_int, c_int, c_float, c_void_p]),
     "mv_sample": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_int, c_void_p]),
     # ... as mv_sample up to chunks, then next_ids, positions, context_lens, stream

@@ -373,15 +373,18 @@ class Ops:
                            rope_table: Optional[torch.Tensor], interleaved: bool,
                            k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
                            block_table: Optional[torch.Tensor], page_size: int,
-                           unit_offset: bool = False) -> None:
+                           unit_offset: bool = False, value_dim: Optional[int] = None) -> None:
         """In place on the rows of ``qkv`` = [q | k | v]: per-head RMSNorm of q and k (when
         weights are given), rotary embedding (when a table is given); k and v are written to
-        the cache pages when pages are given. Without pages the rows hold only q."""
+        the cache pages when pages are given. Without pages the rows hold only q. With
+        ``value_dim`` a value row has that size instead of ``head_dim``, and the rows may hold
+        further columns behind v (nothing touches them)."""
         self._act(qkv, "qkv")
         n = qkv.shape[0]
         store = k_pages is not None
-        width = (num_heads + (2 * num_kv_heads if store else 0)) * head_dim
-        if qkv.dim() != 2 or qkv.shape[1] != width or qkv.stride(1) != 1:
+        vdim = head_dim if value_dim is None else int(value_dim)
+        width = num_heads * head_dim + (num_kv_heads * (head_dim + vdim) if store else 0)
+        if qkv.dim() != 2 or qkv.stride(1) != 1 or (qkv.shape[1] != width if value_dim is None else qkv.shape[1] < width):
             raise KernelLibraryError(f"qk_norm_rope_store: qkv {tuple(qkv.shape)} does not hold {width} columns")
         for t, what in ((positions, "positions"), (token_seq, "token_seq")):
             _dev(t, what)
@@ -404,7 +407,7 @@ class Ops:
             assert v_pages is not None and block_table is not None
             self._act(k_pages, "key pages"); self._act(v_pages, "value pages"); _dev(block_table, "block table")
             if tuple(k_pages.shape[1:]) != (num_kv_heads, page_size, head_dim) or \
-                    tuple(v_pages.shape[1:]) != (num_kv_heads, head_dim, page_size) or \
+                    tuple(v_pages.shape[1:]) != (num_kv_heads, vdim, page_size) or \
                     not k_pages.is_contiguous() or not v_pages.is_contiguous():
                 raise KernelLibraryError(
                     f"qk_norm_rope_store: pages {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not match "
@@ -414,7 +417,19 @@ class Ops:
             bt_width = block_table.shape[1]
         q_dim = num_heads * head_dim
         kv_dim = num_kv_heads * head_dim
-        stride = qkv.stride(0) if n > 1 else width
+        stride = qkv.stride(0) if n > 1 else qkv.shape[1]
+        if store and vdim != head_dim:
+            # values of another size than keys: the keys with the queries, the value rows as a launch of their own
+            self._note("mv_qk_norm_rope_store", n * (2 * q_dim + 2 * kv_dim + 2 * num_kv_heads * vdim) * qkv.element_size()
+                       + (n * rot * 4 if rope_table is not None else 0), 10 * n * (q_dim + kv_dim))
+            self.lib.call("mv_qk_norm_rope_store", qkv.data_ptr(), stride, 0, q_dim, q_dim + kv_dim, positions.data_ptr(),
+                          token_seq.data_ptr(), _ptr(block_table), bt_width, page_size, _ptr(k_pages), _ptr(v_pages), n,
+                          num_heads, num_kv_heads, head_dim, _ptr(q_weight), _ptr(k_weight), wcode, float(eps),
+                          int(unit_offset), _ptr(rope_table), rot, int(interleaved), 2, self.code, self._stream())
+            self.lib.call("mv_store_v_pages", qkv.data_ptr(), stride, q_dim + kv_dim, positions.data_ptr(),
+                          token_seq.data_ptr(), block_table.data_ptr(), bt_width, page_size, v_pages.data_ptr(), n,
+                          num_kv_heads, vdim, self.code, self._stream())
+            return
         # with many tokens the values go to their transposed pages tile by tile, so that
         # neighbouring tokens write neighbouring slots (mode 3); with few, a store per token and head
         mode = 0 if not store else (3 if n >= STORE_V_SPLIT_TOKENS else 1)
@@ -425,6 +440,182 @@ class Ops:
                       page_size, _ptr(k_pages), _ptr(v_pages), n, num_heads, num_kv_heads, head_dim,
                       _ptr(q_weight), _ptr(k_weight), wcode, float(eps), int(unit_offset), _ptr(rope_table), rot,
                       int(interleaved), mode, self.code, self._stream())
+
+    # ------------------------------------------------------------------------------------
+    # parts with a state per request, sandwich norms, capped logits
+    # ------------------------------------------------------------------------------------
+    @staticmethod
+    def _ints(n: int, **tensors) -> None:
+        for what, (t, least) in tensors.items():
+            _dev(t, what)
+            if t.dtype != torch.int32 or t.numel() < least or not t.is_contiguous():
+                raise KernelLibraryError(f"{what} must be contiguous int32 with at least {least} elements")
+
+    def token_shift(self, h: torch.Tensor, mix: torch.Tensor, state: torch.Tensor, token_seq: torch.Tensor,
+                    cu_seqlens: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor) -> None:
+        """out[t] = h[t] + (h[t-1] - h[t]) * mix; the row in front of a request's first row of the step
+        is state[slot], which then takes the request's last row. h, out [n, w]; state [slots, w]."""
+        self._act(h, "shift input"); self._act(out, "shift output"); self._act(state, "shift state"); _dev(mix, "shift weight")
+        n, w = h.shape
+        if out.shape != h.shape or h.stride(1) != 1 or out.stride(1) != 1 or out.data_ptr() == h.data_ptr():
+            raise KernelLibraryError("token_shift: input and output must be two [n, w] buffers")
+        if state.dim() != 2 or state.shape[1] != w or not state.is_contiguous() or mix.numel() != w or not mix.is_contiguous():
+            raise KernelLibraryError(f"token_shift: state {tuple(state.shape)} / weight {tuple(mix.shape)} do not fit rows of {w}")
+        self._ints(n, token_seq=(token_seq, n), cu_seqlens=(cu_seqlens, 2), state_slots=(state_slots, 1))
+        self._note("mv_token_shift", 2 * self._size(h) + self._size(out), 3 * n * w)
+        self.lib.call("mv_token_shift", h.data_ptr(), h.stride(0) if n > 1 else w, out.data_ptr(),
+                      out.stride(0) if n > 1 else w, mix.data_ptr(), _weight_code(mix, "shift weight"), state.data_ptr(),
+                      token_seq.data_ptr(), cu_seqlens.data_ptr(), state_slots.data_ptr(), n, w, self.code, self._stream())
+
+    def delta_prepare(self, packed: torch.Tensor, heads: int, dim: int, rank: int, w2: torch.Tensor, w0: torch.Tensor,
+                      a_bias: torch.Tensor, decay_rate: float, key_eps: float, token_seq: torch.Tensor,
+                      coef: torch.Tensor) -> None:
+        """From rows [r | k | v | g | a | w1] (heads*dim columns each, ``rank`` for w1) the float32
+        coefficients of the delta rule, coef [3, n, heads*dim]: the decay
+        exp(-decay_rate * sigmoid(w2 tanh(w1) + w0)), rate * unit key with rate = sigmoid(a + a_bias),
+        and the unit key k / sqrt(sum(k^2) + key_eps) of each head."""
+        self._act(packed, "delta rows")
+        n, inner = packed.shape[0], heads * dim
+        if packed.dim() != 2 or packed.stride(1) != 1 or packed.shape[1] < 5 * inner + rank:
+            raise KernelLibraryError(f"delta_prepare: rows {tuple(packed.shape)} do not hold 5 x {inner} + {rank} columns")
+        if coef.dtype != torch.float32 or tuple(coef.shape) != (3, n, inner) or not coef.is_contiguous():
+            raise KernelLibraryError(f"delta_prepare: coefficients must be float32 [3, {n}, {inner}]")
+        for t, shape, what in ((w2, (inner, rank), "w2"), (w0, (inner,), "w0"), (a_bias, (inner,), "a_bias")):
+            _dev(t, what)
+            if tuple(t.shape) != shape or not t.is_contiguous() or t.dtype != w2.dtype:
+                raise KernelLibraryError(f"delta_prepare: {what} must be a contiguous {shape} tensor of w2's dtype")
+        self._ints(n, token_seq=(token_seq, n))
+        self._note("mv_delta_prepare", n * (2 * inner + rank) * packed.element_size() + self._size(w2, coef), 2 * n * inner * rank)
+        self.lib.call("mv_delta_prepare", packed.data_ptr(), packed.stride(0) if n > 1 else packed.shape[1], n, heads, dim,
+                      rank, w2.data_ptr(), w0.data_ptr(), a_bias.data_ptr(), _weight_code(w2, "w2"), float(decay_rate),
+                      float(key_eps), token_seq.data_ptr(), coef.data_ptr(), self.code, self._stream())
+
+    def delta_scan(self, packed: torch.Tensor, coef: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor,
+                   state_slots: torch.Tensor, n_seqs: int, heads: int, dim: int, out: torch.Tensor) -> None:
+        """The delta rule over the step's rows, request by request (rows cu_seqlens[s] .. cu_seqlens[s+1]
+        of request s, state row state_slots[s]): S <- diag(w) S - (a*u)(u^T S) + k v^T, out = S^T r, with
+        r, k, v from the packed rows and w, a*u, u from ``coef``. state float32 [slots, heads, dim, dim] is
+        read and left advanced; out float32 [n, heads*dim]."""
+        self._act(packed, "delta rows")
+        n, inner = packed.shape[0], heads * dim
+        if coef.dtype != torch.float32 or tuple(coef.shape) != (3, n, inner) or not coef.is_contiguous():
+            raise KernelLibraryError(f"delta_scan: coefficients must be float32 [3, {n}, {inner}]")
+        if out.dtype != torch.float32 or tuple(out.shape) != (n, inner) or not out.is_contiguous():
+            raise KernelLibraryError(f"delta_scan: the output must be float32 [{n}, {inner}]")
+        _dev(state, "delta state")
+        if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, dim) or not state.is_contiguous():
+            raise KernelLibraryError(f"delta_scan: the state must be float32 [slots, {heads}, {dim}, {dim}]")
+        if packed.dim() != 2 or packed.stride(1) != 1 or packed.shape[1] < 3 * inner:
+            raise KernelLibraryError(f"delta_scan: rows {tuple(packed.shape)} do not hold r, k and v")
+        self._ints(n, cu_seqlens=(cu_seqlens, n_seqs + 1), state_slots=(state_slots, n_seqs))
+        self._note("mv_delta_scan", 3 * n * inner * packed.element_size() + self._size(coef, out)
+                   + 2 * min(n_seqs, max(n, 1)) * inner * dim * 4, 8 * n * inner * dim)
+        self.lib.call("mv_delta_scan", packed.data_ptr(), packed.stride(0) if n > 1 else packed.shape[1], coef.data_ptr(),
+                      state.data_ptr(), cu_seqlens.data_ptr(), state_slots.data_ptr(), n_seqs, n, heads, dim,
+                      out.data_ptr(), self.code, self._stream())
+
+    def delta_finish(self, raw: torch.Tensor, packed: torch.Tensor, weight: torch.Tensor, heads: int, dim: int,
+                     eps: float, out: torch.Tensor) -> None:
+        """out = raw / rms(raw over each head) * weight * sigmoid(g), g the fourth block of the packed rows."""
+        self._act(packed, "delta rows"); self._act(out, "delta output"); _dev(weight, "delta norm weight")
+        n, inner = packed.shape[0], heads * dim
+        if raw.dtype != torch.float32 or tuple(raw.shape) != (n, inner) or not raw.is_contiguous():
+            raise KernelLibraryError(f"delta_finish: the scan's output must be float32 [{n}, {inner}]")
+        if tuple(out.shape) != (n, inner) or out.stride(1) != 1 or packed.shape[1] < 4 * inner or weight.numel() != inner \
+                or not weight.is_contiguous():
+            raise KernelLibraryError("delta_finish: operands do not fit")
+        self._note("mv_delta_finish", self._size(raw, out) + n * inner * packed.element_size(), 8 * n * inner)
+        self.lib.call("mv_delta_finish", raw.data_ptr(), packed.data_ptr(), packed.stride(0) if n > 1 else packed.shape[1],
+                      weight.data_ptr(), _weight_code(weight, "delta norm weight"), n, heads, dim, float(eps),
+                      out.data_ptr(), out.stride(0) if n > 1 else inner, self.code, self._stream())
+
+    def norm_add_norm(self, y: torch.Tensor, norm_y, resid: torch.Tensor, norm_next, out: Optional[torch.Tensor]) -> None:
+        """resid += rmsnorm(y) * w (``norm_y`` = (weight, eps, unit_offset)); with ``norm_next`` of the same
+        form, out = rmsnorm(resid) * w'. The sum stays float32 in between."""
+        self._act(y, "sublayer output"); _dev(resid, "residual")
+        n, h = resid.shape
+        if resid.dtype != torch.float32 or not resid.is_contiguous() or tuple(y.shape) != (n, h) or y.stride(1) != 1:
+            raise KernelLibraryError("norm_add_norm: a float32 residual [n, h] and an output of the same shape are needed")
+        wa, eps_a, unit_a = norm_y
+        _dev(wa, "norm weight")
+        if wa.numel() != h or not wa.is_contiguous():
+            raise KernelLibraryError(f"norm_add_norm: weight of {wa.numel()} elements for rows of {h}")
+        wb, eps_b, unit_b, wb_code = None, 1.0, False, DTYPE_F32
+        if out is not None:
+            if norm_next is None:
+                raise KernelLibraryError("norm_add_norm: an output needs the second norm")
+            self._act(out, "norm output")
+            wb, eps_b, unit_b = norm_next
+            _dev(wb, "norm weight")
+            wb_code = _weight_code(wb, "norm weight")
+            if wb.numel() != h or not wb.is_contiguous() or tuple(out.shape) != (n, h) or not out.is_contiguous():
+                raise KernelLibraryError("norm_add_norm: the second norm's weight or output does not fit")
+        self._note("mv_norm_add_norm", self._size(y, out) + 2 * self._size(resid), 8 * n * h)
+        self.lib.call("mv_norm_add_norm", y.data_ptr(), y.stride(0) if n > 1 else h, wa.data_ptr(),
+                      _weight_code(wa, "norm weight"), float(eps_a), int(unit_a), resid.data_ptr(), _ptr(wb), wb_code,
+                      float(eps_b), int(unit_b), _ptr(out), n, h, self.code, self._stream())
+
+    def soft_cap(self, logits: torch.Tensor, cap: float) -> None:
+        """In place on float32 [rows, cols]: x <- cap * tanh(x / cap)."""
+        _dev(logits, "logits")
+        if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+            raise KernelLibraryError("soft_cap: float32 rows with a contiguous last dimension are needed")
+        rows, cols = logits.shape
+        if rows == 0:
+            return
+        self._note("mv_soft_cap", 2 * self._size(logits), 4 * rows * cols)
+        self.lib.call("mv_soft_cap", logits.data_ptr(), logits.stride(0) if rows > 1 else cols, rows, cols, float(cap),
+                      self._stream())
+
+    def attention_sigmoid(self, q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                          block_table: torch.Tensor, page_size: int, positions: torch.Tensor, token_seq: torch.Tensor,
+                          num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float,
+                          chunk: Optional[int], window: Optional[int], bias: Optional[torch.Tensor],
+                          gate: Optional[torch.Tensor], plan: Optional["AttentionPlan"] = None) -> None:
+        """Causal attention with sigmoid weights over the paged cache: the query at position p sees the
+        keys of its request from max(start of p's chunk, p - window, 0) to p, each with the weight
+        sigmoid(q.k * scale + bias[head]), not normalised. q [n, >= H*D] rows, out [n, H*Dv]; bias float32
+        [H] or None; gate [n, >= H] rows of the activation type or None (head h's output times
+        sigmoid(gate[t, h]))."""
+        self._act(q, "queries"); self._act(out, "attention output")
+        self._act(k_pages, "key pages"); self._act(v_pages, "value pages")
+        n = q.shape[0]
+        if q.dim() != 2 or q.shape[1] < num_heads * head_dim or q.stride(1) != 1 \
+                or tuple(out.shape) != (n, num_heads * value_dim) or out.stride(1) != 1:
+            raise KernelLibraryError(f"attention_sigmoid: q {tuple(q.shape)} / out {tuple(out.shape)} do not hold "
+                                     f"{num_heads} heads of {head_dim} / {value_dim}")
+        if tuple(k_pages.shape[1:]) != (num_kv_heads, page_size, head_dim) or \
+                tuple(v_pages.shape[1:]) != (num_kv_heads, value_dim, page_size) or \
+                not k_pages.is_contiguous() or not v_pages.is_contiguous():
+            raise KernelLibraryError(f"attention_sigmoid: pages {tuple(k_pages.shape)} / {tuple(v_pages.shape)} have the "
+                                     f"wrong layout for {num_kv_heads} heads of {head_dim} / {value_dim}, page {page_size}")
+        self._ints(n, positions=(positions, n), token_seq=(token_seq, n))
+        _dev(block_table, "block table")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+            raise KernelLibraryError("attention_sigmoid: the block table must be a contiguous int32 matrix")
+        if num_heads % num_kv_heads:
+            raise KernelLibraryError(f"attention_sigmoid: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if bias is not None:
+            _dev(bias, "score bias")
+            if bias.dtype != torch.float32 or bias.numel() != num_heads or not bias.is_contiguous():
+                raise KernelLibraryError(f"attention_sigmoid: the score bias must be float32 [{num_heads}]")
+        gate_stride = 0
+        if gate is not None:
+            self._act(gate, "head gates")
+            if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < num_heads or gate.stride(1) != 1:
+                raise KernelLibraryError(f"attention_sigmoid: gates {tuple(gate.shape)} do not hold {num_heads} per row")
+            gate_stride = gate.stride(0) if n > 1 else gate.shape[1]
+        if n == 0:
+            return
+        c = 0 if chunk is None else int(chunk)
+        w = -1 if window is None else int(window)
+        qs = q.stride(0) if n > 1 else q.shape[1]
+        os_ = out.stride(0) if n > 1 else num_heads * value_dim
+        self._note("mv_attention_sigmoid", self._size(q, out), 0)
+        self.lib.call("mv_attention_sigmoid_ref", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
+                      v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size, positions.data_ptr(),
+                      token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim, value_dim, float(scale), c, w,
+                      _ptr(bias), _ptr(gate), gate_stride, self.code, self._stream())
 
     def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
         """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""

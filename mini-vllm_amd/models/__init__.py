@@ -1,4 +1,5 @@
 from .registry import (Architecture, config_from_dict, get_architecture, load_config, register_architecture,
                        registered_architectures, unregister_architecture)
 from . import qwen3  # registers "Qwen3ForCausalLM"
+from . import bolapel  # registers "Bolapel"
 from .causal_lm import CausalLM, expected_tensors

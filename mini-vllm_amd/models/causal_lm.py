@@ -43,6 +43,8 @@ def plan_tensors(plan: ModelPlan) -> List[Tuple[TensorLocation, TensorDecl]]:
         for slot, nspec in layer.norms:
             for name, decl in NORMS.get(nspec.kind).tensors(nspec).items():
                 out.append((TensorLocation(i, f"norm.{slot}", name), decl))
+        for name, decl in getattr(block_cls, "tensors", lambda spec: {})(layer.block).items():
+            out.append((TensorLocation(i, "block", name), decl))
         if layer.mixer is not None:
             for name, decl in MIXERS.get(layer.mixer.kind).tensors(layer.mixer).items():
                 out.append((TensorLocation(i, "mixer", name), decl))
@@ -116,7 +118,13 @@ class CausalLM:
                 ffn_cls = FEED_FORWARDS.get(layer.ffn.kind)
                 ffn = ffn_cls(layer.ffn, fetch(i, "ffn", ffn_cls.tensors(layer.ffn)), rt)
             self.mixers.append(mixer)
-            self.blocks.append(BLOCKS.get(layer.block.kind)(layer.block, norms, mixer, ffn))
+            block_cls = BLOCKS.get(layer.block.kind)
+            if getattr(block_cls, "wants_runtime", False):
+                block = block_cls(layer.block, norms, mixer, ffn,
+                                  tensors=fetch(i, "block", block_cls.tensors(layer.block)), rt=rt)
+            else:
+                block = block_cls(layer.block, norms, mixer, ffn)
+            self.blocks.append(block)
             parts = [mixer, ffn, kwargs.get("position")] + list(norms.values())
             self.graph_safe = self.graph_safe and all(getattr(p, "graph_safe", True) for p in parts if p is not None)
         self.graph_safe = self.graph_safe and all(getattr(p, "graph_safe", True)
@@ -138,11 +146,20 @@ class CausalLM:
             needs.append(need)
         return needs
 
-    def state_shapes(self) -> List[Optional[Tuple[Tuple[int, ...], torch.dtype]]]:
+    def state_shapes(self) -> List[Optional[Dict[str, Tuple[Tuple[int, ...], torch.dtype]]]]:
+        """Per call: name -> (shape, dtype) of every fixed-size state a request holds for it (its
+        mixer's and its block arrangement's), None if it holds none. A dtype of None stands for the
+        activation type."""
         out = []
         for call in self.plan.calls:
-            spec = self.plan.layers[call.layer].mixer
-            out.append(None if spec is None else MIXERS.get(spec.kind).state_shape(spec))
+            layer = self.plan.layers[call.layer]
+            shapes = {}
+            if layer.mixer is not None:
+                shapes.update(MIXERS.get(layer.mixer.kind).state_shapes(layer.mixer))
+            block_cls = BLOCKS.get(layer.block.kind)
+            shapes.update(getattr(block_cls, "state_shapes", lambda spec: {})(layer.block))
+            out.append({name: (tuple(dims), self.rt.dtype if dt is None else dt)
+                        for name, (dims, dt) in shapes.items()} or None)
         return out
 
     # ------------------------------------------------------------------------------------

@@ -10,7 +10,7 @@ the plan's logical tensor names to the names on disk.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, FrozenSet, List, Type
+from typing import Any, Callable, Dict, FrozenSet, List, Optional, Type
 
 from ..config.model_config import ConfigError, ModelConfig, architecture_name, read_config_json
 from ..parts.plan import ModelPlan, TensorLocation
@@ -25,6 +25,9 @@ class Architecture:
     # names that may be present in the model folder without being used (e.g. a stored copy of
     # a tied output head)
     ignorable: Callable[[ModelConfig], FrozenSet[str]] = lambda config: frozenset()
+    # (config, tensor source) -> config: fills in sizes that config.json leaves to the shapes of the
+    # stored tensors; None when config.json states everything
+    complete: Optional[Callable[[ModelConfig, Any], ModelConfig]] = None
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}

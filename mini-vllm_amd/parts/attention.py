@@ -8,15 +8,22 @@ itself (attention.py:56-60); None sees all.
 
 Every size is a parameter of the spec. q, k and v are packed into one matrix product; the
 per-head norms, the rotary embedding and the cache write are one kernel.
+
+Beyond the reference's layer the spec has, each off by default: values of another size than keys
+(``value_dim``); ``chunk``: a query sees only the keys of its own chunk of the sequence (positions
+with equal ``position // chunk``, counted from the sequence's start); ``weighting = "sigmoid"``: the
+weight of a visible key is sigmoid(score * scale + score_bias[head]) and the weights are not
+normalised over the keys; ``head_gate``: head h's output is multiplied by sigmoid(W_gate x)[h], one
+number per head, read from the same packed product as q, k and v.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Optional
+from typing import Dict, Optional, Tuple
 
 import torch
 
-from .base import CacheNeed, KeepAll, KeepWindow, KeyValueNeed, Mixer, PartSpec, Runtime, TensorDecl, register_mixer
+from .base import CacheNeed, KeepAll, KeepChunks, KeepWindow, KeyValueNeed, Mixer, PartSpec, Runtime, TensorDecl, register_mixer
 
 
 @dataclass(frozen=True)
@@ -33,6 +40,15 @@ class AttentionSpec(PartSpec):
     window: Optional[int] = None
     position: Optional[PartSpec] = None
     shares_kv: bool = False        # no k/v of its own: reads the cache of the call named by the plan
+    value_dim: Optional[int] = None          # None: head_dim
+    weighting: str = "softmax"               # or "sigmoid"
+    score_bias: bool = False                 # a learned number per head added to the scaled score (sigmoid weighting)
+    chunk: Optional[int] = None
+    head_gate: bool = False
+    # chunk sizes of every call that reads this call's cache, its own among them (they decide how long
+    # pages stay); empty: its own ``chunk`` alone. ``cache_keeps_all``: some reader sees all keys.
+    cache_chunks: Tuple[int, ...] = ()
+    cache_keeps_all: bool = False
 
     @property
     def q_dim(self) -> int:
@@ -41,6 +57,24 @@ class AttentionSpec(PartSpec):
     @property
     def kv_dim(self) -> int:
         return self.num_kv_heads * self.head_dim
+
+    @property
+    def v_head_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
+
+    @property
+    def v_dim(self) -> int:
+        return self.num_kv_heads * self.v_head_dim
+
+    @property
+    def out_dim(self) -> int:
+        return self.num_heads * self.v_head_dim
+
+    @property
+    def plain(self) -> bool:
+        """The reference's layer: softmax over all keys or a window, values as large as keys."""
+        return (self.weighting == "softmax" and self.chunk is None and self.value_dim in (None, self.head_dim)
+                and not self.head_gate and not self.score_bias)
 
 
 @register_mixer(AttentionSpec.kind)
@@ -51,10 +85,14 @@ class Attention(Mixer):
 
     @classmethod
     def tensors(cls, spec: AttentionSpec) -> Dict[str, TensorDecl]:
-        t = {"q": TensorDecl((spec.q_dim, spec.hidden_size)), "o": TensorDecl((spec.hidden_size, spec.q_dim))}
+        t = {"q": TensorDecl((spec.q_dim, spec.hidden_size)), "o": TensorDecl((spec.hidden_size, spec.out_dim))}
         if not spec.shares_kv:
             t["k"] = TensorDecl((spec.kv_dim, spec.hidden_size))
-            t["v"] = TensorDecl((spec.kv_dim, spec.hidden_size))
+            t["v"] = TensorDecl((spec.v_dim, spec.hidden_size))
+        if spec.score_bias:
+            t["score_bias"] = TensorDecl((spec.num_heads,), init="zeros_normal")
+        if spec.head_gate:
+            t["head_gate"] = TensorDecl((spec.num_heads, spec.hidden_size))
         if spec.bias:
             t["q_bias"] = TensorDecl((spec.q_dim,), init="zeros_normal")
             t["o_bias"] = TensorDecl((spec.hidden_size,), init="zeros_normal")
@@ -71,24 +109,36 @@ class Attention(Mixer):
     def cache_need(cls, spec: AttentionSpec) -> Optional[CacheNeed]:
         if spec.shares_kv:
             return None
-        return KeyValueNeed(retention=KeepAll() if spec.window is None else KeepWindow(spec.window),
-                            num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim)
+        if spec.chunk is not None or spec.cache_chunks:
+            sizes = tuple(sorted(set(spec.cache_chunks or (spec.chunk,))))
+            retention = KeepAll() if spec.cache_keeps_all else KeepChunks(sizes)
+        else:
+            retention = KeepAll() if (spec.window is None or spec.cache_keeps_all) else KeepWindow(spec.window)
+        return KeyValueNeed(retention=retention, num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim,
+                            value_dim=spec.value_dim)
 
     def __init__(self, spec: AttentionSpec, tensors: Dict[str, torch.Tensor], rt: Runtime,
                  position: Optional[object] = None):
         if spec.num_heads % spec.num_kv_heads:
             raise ValueError(f"{spec.num_heads} query heads are not a multiple of {spec.num_kv_heads} kv heads")
+        if spec.weighting not in ("softmax", "sigmoid"):
+            raise ValueError(f"attention weighting must be 'softmax' or 'sigmoid', got {spec.weighting!r}")
+        if not spec.plain and (spec.weighting != "sigmoid" or spec.bias):
+            raise NotImplementedError("chunks, a value size of its own, a score bias and head gates are built for "
+                                      "sigmoid weighting without projection biases")
         self.spec = spec
         self.rt = rt
         parts = ["q"] if spec.shares_kv else ["q", "k", "v"]
+        if spec.head_gate:
+            parts = parts + ["head_gate"]
         dtypes = {tensors[p].dtype for p in parts}
         if len(dtypes) != 1:
             raise ValueError(f"q, k and v projections are stored in different dtypes {dtypes}; cannot pack them")
-        self.w_qkv = tensors["q"] if spec.shares_kv else torch.cat([tensors[p] for p in parts], dim=0).contiguous()
+        self.w_qkv = tensors["q"] if len(parts) == 1 else torch.cat([tensors[p] for p in parts], dim=0).contiguous()
         self.b_qkv = None
         self.b_o = None
         if spec.bias:
-            self.b_qkv = tensors["q_bias"] if spec.shares_kv else torch.cat(
+            self.b_qkv = tensors["q_bias"] if len(parts) == 1 else torch.cat(
                 [tensors[p + "_bias"] for p in parts], dim=0).contiguous()
             self.b_o = tensors["o_bias"]
         self.w_o = tensors["o"]
@@ -98,13 +148,29 @@ class Attention(Mixer):
         self.rotary = position.rotary() if position is not None else None
         if position is not None and self.rotary is None and not hasattr(position, "apply"):
             raise ValueError("a position encoding must offer rotary() or apply()")
-        self.width = spec.q_dim + (0 if spec.shares_kv else 2 * spec.kv_dim)
+        self.width = spec.q_dim + (0 if spec.shares_kv else spec.kv_dim + spec.v_dim)
+        self.gate_off = self.width                        # the head gates come last in the packed rows
+        if spec.head_gate:
+            self.width += spec.num_heads
+        self.score_bias = tensors.get("score_bias")
+        if self.score_bias is not None:
+            self.score_bias = self.score_bias.to(torch.float32)
+        if self.w_qkv.shape[0] != self.width:
+            raise ValueError(f"the packed projection has {self.w_qkv.shape[0]} rows, expected {self.width}")
+        if not spec.plain and self.width % 8:
+            # rows of the packed product keep a pitch of a multiple of 8 elements (zero rows at the end)
+            pad = (-self.width) % 8
+            self.w_qkv = torch.cat([self.w_qkv, torch.zeros((pad, spec.hidden_size), dtype=self.w_qkv.dtype,
+                                                            device=self.w_qkv.device)], dim=0).contiguous()
+            self.width += pad
 
     def first_product(self):
         return self.w_qkv.shape[0], self.w_qkv.shape[1], False
 
     def forward(self, x: torch.Tensor, ctx, call: int, fold=None) -> torch.Tensor:
         spec, rt, ops = self.spec, self.rt, self.rt.ops
+        if not spec.plain:
+            return self._forward_sigmoid(x, ctx, call)
         n = x.shape[0]
         ws = rt.workspace
         qkv = ws.get("attn.qkv", (n, self.width), rt.dtype)
@@ -141,3 +207,28 @@ class Attention(Mixer):
         y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
         # (the sums of a product whose K was split may be left to the next norm)
         return ops.gemm(attn, self.w_o, y, self.b_o, defer_sum=True, fold=fold) or y
+
+    def _forward_sigmoid(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
+        """Sigmoid weighting (chunks, a window or all keys; values of any size; score bias; head gates)."""
+        spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
+        n = x.shape[0]
+        packed = ws.get("attn.qkv", (n, self.width), rt.dtype)
+        ops.gemm(x, self.w_qkv, packed)
+        kv = ctx.kv(call)
+        table, interleaved = (self.rotary if self.rotary is not None else (None, False))
+        if self.position is not None and self.rotary is None:
+            raise NotImplementedError("sigmoid attention takes its rotation from a rotary table")
+        own = not spec.shares_kv
+        ops.qk_norm_rope_store(
+            packed, spec.num_heads, spec.num_kv_heads, spec.head_dim, ctx.positions, ctx.token_seq,
+            self.q_norm, self.k_norm, spec.qk_norm_eps, table, interleaved,
+            kv.k_pages if own else None, kv.v_pages if own else None, kv.block_table if own else None, kv.page_size,
+            value_dim=spec.v_head_dim)
+        attn = ws.get("attn.out", (n, spec.out_dim), rt.dtype)
+        gate = packed[:, self.gate_off:self.gate_off + spec.num_heads] if spec.head_gate else None
+        ops.attention_sigmoid(packed[:, :spec.q_dim], attn, kv.k_pages, kv.v_pages, kv.block_table, kv.page_size,
+                              ctx.positions, ctx.token_seq, spec.num_heads, spec.num_kv_heads, spec.head_dim,
+                              spec.v_head_dim, spec.scale, spec.chunk, spec.window, self.score_bias, gate,
+                              plan=ctx.attention_plan)
+        y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
+        return ops.gemm(attn, self.w_o, y, self.b_o, defer_sum=True) or y

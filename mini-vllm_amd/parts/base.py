@@ -121,6 +121,34 @@ class KeepWindow(Retention):
         return min(-(-length // page_size), (self.window + max(1, portion)) // page_size + 2)
 
 
+@dataclass(frozen=True)
+class KeepChunks(Retention):
+    """For mixers whose queries see only their own chunk of the sequence (positions p with equal
+    ``p // size``): a page stays while any of the ``sizes`` (one per call that reads the cache) still
+    has a chunk that reaches into it; pages in front of the oldest such chunk go back to the pool."""
+    sizes: Tuple[int, ...] = ()
+
+    def __post_init__(self):
+        if not self.sizes or any(s < 1 for s in self.sizes):
+            raise ValueError(f"chunk sizes must be >= 1, got {self.sizes}")
+
+    def first_kept_page(self, next_position: int, page_size: int) -> int:
+        return min(next_position // s * s for s in self.sizes) // page_size
+
+    def first_kept_pages(self, next_positions, page_size: int):
+        import numpy as np
+        p = np.asarray(next_positions, dtype=np.int64)
+        first = p // self.sizes[0] * self.sizes[0]
+        for s in self.sizes[1:]:
+            first = np.minimum(first, p // s * s)
+        return first // page_size
+
+    def most_pages_held(self, length: int, page_size: int, portion: int) -> Optional[int]:
+        # while a portion runs: the chunk its first token stands in, the portion itself, and the
+        # two pages that the ends of that range may only touch
+        return min(-(-length // page_size), (max(self.sizes) + max(1, portion)) // page_size + 2)
+
+
 class CacheNeed:
     """Paged memory a mixer needs for each token of a request: which tensors a page consists of
     and how long positions are kept. The executor allocates ``[pages, *shape]`` per named tensor
@@ -165,9 +193,11 @@ class KeyValueNeed(CacheNeed):
     retention: Retention
     num_kv_heads: int
     head_dim: int
+    value_dim: Optional[int] = None        # size of a value row where it differs from a key's
 
     def page_shapes(self, page_size: int) -> Dict[str, Tuple[int, ...]]:
-        return {"k": (self.num_kv_heads, page_size, self.head_dim), "v": (self.num_kv_heads, self.head_dim, page_size)}
+        vd = self.head_dim if self.value_dim is None else self.value_dim
+        return {"k": (self.num_kv_heads, page_size, self.head_dim), "v": (self.num_kv_heads, vd, page_size)}
 
 
 # ---------------------------------------------------------------------------------------
@@ -283,11 +313,15 @@ class HiddenStream:
     defer_sum=True)`` returned in its place (an output whose partial sums the norm's kernel adds
     up itself; it has ``shape``, ``materialize()`` and ``discard()``)."""
 
-    __slots__ = ("resid", "delta", "spare", "weighted")
+    __slots__ = ("resid", "delta", "spare", "weighted", "normed")
 
     def __init__(self, resid: torch.Tensor, spare: Optional[torch.Tensor] = None):
         self.resid = resid
         self.delta: Optional[torch.Tensor] = None
+        # (norm, rows): the rows of ``resid`` as ``norm`` leaves them, computed already by the kernel
+        # that made ``resid`` (a block that closes a sublayer and opens the next in one launch);
+        # that norm takes them from here instead of running
+        self.normed = None
         # rows that the last product already added to ``resid`` and left half normalised for the
         # norm that comes next (see NormFold); that norm takes them from here
         self.weighted = None
@@ -435,6 +469,13 @@ class Mixer(Part):
         """Shape and dtype of the fixed-size state each request holds for this mixer."""
         return None
 
+    @classmethod
+    def state_shapes(cls, spec) -> Dict[str, Tuple[Tuple[int, ...], torch.dtype]]:
+        """The same by name, for a mixer with several state tensors (``ctx.state(call, name)``); the
+        default is the one of ``state_shape`` under the name "state"."""
+        one = cls.state_shape(spec)
+        return {} if one is None else {"state": one}
+
     def forward(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
         raise NotImplementedError
 
@@ -472,9 +513,23 @@ class Block:
     output (``entry_norm()``, ``entry_part()``), or None. It may offer that norm to its last part
     (``NormFold``)."""
     accepts_next_norm: ClassVar[bool] = False
+    # a block with tensors or state of its own is also given ``tensors=`` (logical name -> device
+    # tensor) and ``rt=`` when it is built
+    wants_runtime: ClassVar[bool] = False
 
     def __init__(self, spec, norms: Dict[str, Norm], mixer: Mixer, ffn: FeedForward):
         raise NotImplementedError
+
+    @classmethod
+    def tensors(cls, spec) -> Dict[str, TensorDecl]:
+        """Tensors of the arrangement itself (role "block"), by logical name."""
+        return {}
+
+    @classmethod
+    def state_shapes(cls, spec) -> Dict[str, Tuple[Tuple[int, ...], torch.dtype]]:
+        """Fixed-size state each request holds for every call of a layer so arranged, by name
+        (``ctx.state(call, name)``)."""
+        return {}
 
     def entry_norm(self) -> Optional["Norm"]:
         """The norm this block applies to the stream before anything else, if it starts with one."""

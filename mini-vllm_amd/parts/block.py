@@ -8,6 +8,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Dict, Optional, Tuple
 
+import torch
+
 from .base import Block, FeedForward, HiddenStream, Mixer, Norm, PartSpec, register_block
 
 
@@ -60,3 +62,91 @@ class PreNormBlock(Block):
             stream.delta, stream.weighted = None, out      # already added to the residual
         else:
             stream.delta = out
+
+
+@dataclass(frozen=True)
+class SandwichBlockSpec(PartSpec):
+    """A norm in front of and behind every sublayer; ``token_shift`` mixes each row of the mixer's
+    input with the row of the token before it (``hidden_size`` is the width of those rows)."""
+    kind = "sandwich"
+    hidden_size: int = 0
+    token_shift: bool = False
+
+
+@register_block(SandwichBlockSpec.kind)
+class SandwichBlock(Block):
+    """x = x + norm_mixer_out(mixer(shift(norm_mixer(x)))); x = x + norm_ffn_out(ffn(norm_ffn(x))).
+
+    ``shift``: h[t] <- h[t] + (h[t-1] - h[t]) * mix, element by element, with the rows as the norm
+    left them; the row in front of a request's first token is zero, and the last row of a step is
+    kept as the request's state (``shift.last``) for its next step. A layer without a feed-forward
+    has only the first half.
+
+    The norm behind a sublayer, the residual add and the norm in front of the next sublayer are
+    one kernel when both norms are plain scaled RMS norms (``Norm.as_scaled_rms``): the sum never
+    leaves float32 and the next norm finds its rows in ``stream.normed``."""
+    norm_slots: Tuple[str, ...] = ("norm1", "norm1b", "norm2", "norm2b")
+    accepts_next_norm = True
+    wants_runtime = True
+
+    @classmethod
+    def slots_for(cls, has_ffn: bool) -> Tuple[str, ...]:
+        return cls.norm_slots if has_ffn else cls.norm_slots[:2]
+
+    @classmethod
+    def tensors(cls, spec: SandwichBlockSpec):
+        from .base import TensorDecl
+        return {"shift": TensorDecl((spec.hidden_size,), init="zeros_normal")} if spec.token_shift else {}
+
+    @classmethod
+    def state_shapes(cls, spec: SandwichBlockSpec):
+        # the mixer's input row of the request's last token, in the activation type (None: the runtime's)
+        return {"shift.last": ((spec.hidden_size,), None)} if spec.token_shift else {}
+
+    def __init__(self, spec: SandwichBlockSpec, norms: Dict[str, Norm], mixer: Mixer, ffn: FeedForward,
+                 tensors=None, rt=None):
+        self.spec, self.rt = spec, rt
+        self.mixer, self.ffn = mixer, ffn
+        self.norm_in, self.norm_out = norms["norm1"], norms["norm1b"]
+        self.norm_ffn_in, self.norm_ffn_out = (norms["norm2"], norms["norm2b"]) if ffn is not None else (None, None)
+        self.shift = (tensors or {}).get("shift")
+        if spec.token_shift and (self.shift is None or rt is None):
+            raise ValueError("a block with token shift needs its 'shift' tensor and the runtime")
+
+    def entry_norm(self) -> Norm:
+        return self.norm_in
+
+    def entry_part(self):
+        return None            # the rows pass through the shift first: no product takes the norm over
+
+    def forward(self, stream: HiddenStream, ctx, call: int, next_norm: Optional[Norm] = None, next_part=None) -> None:
+        h = self.norm_in.forward(stream, ctx)
+        if self.shift is not None:
+            mixed = self.rt.workspace.get("shift.out", tuple(h.shape), h.dtype)
+            self.rt.ops.token_shift(h, self.shift, ctx.state(call, "shift.last"), ctx.token_seq, ctx.cu_seqlens,
+                                    ctx.state_slots, mixed)
+            h = mixed
+        y = self.mixer.forward(h, ctx, call)
+        self._close(stream, ctx, y, self.norm_out, self.norm_ffn_in if self.ffn is not None else next_norm)
+        if self.ffn is not None:
+            h = self.norm_ffn_in.forward(stream, ctx)
+            y = self.ffn.forward(h, ctx)
+            self._close(stream, ctx, y, self.norm_ffn_out, next_norm)
+
+    def _close(self, stream: HiddenStream, ctx, y, norm_out: Norm, norm_next: Optional[Norm]) -> None:
+        """resid += norm_out(y); the rows of ``norm_next`` are left in the stream when it can ride along."""
+        if not isinstance(y, torch.Tensor):
+            y = y.materialize()
+        out_form = norm_out.as_scaled_rms()
+        next_form = norm_next.as_scaled_rms() if norm_next is not None else None
+        if out_form is None:
+            tmp = self.rt.workspace.get("sandwich.delta", tuple(y.shape), y.dtype)
+            norm_out.apply(y, tmp)
+            stream.delta = tmp           # the next norm (or the model's last) adds it
+            return
+        rows = None
+        if next_form is not None:
+            rows = self.rt.workspace.get("normed", tuple(y.shape), y.dtype)
+        self.rt.ops.norm_add_norm(y, out_form, stream.resid, next_form, rows)
+        stream.delta = None
+        stream.normed = (norm_next, rows) if rows is not None else None

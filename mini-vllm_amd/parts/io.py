@@ -11,11 +11,12 @@ another registered class; the model code does not change.
 """
 from __future__ import annotations
 
+from dataclasses import dataclass
 from typing import Dict
 
 import torch
 
-from .base import Embedding, Head, Runtime, TensorDecl, register_embedding, register_head
+from .base import Embedding, Head, PartSpec, Runtime, TensorDecl, register_embedding, register_head
 from .plan import EmbeddingSpec, HeadSpec
 
 
@@ -51,4 +52,28 @@ class LinearHead(Head):
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         logits = self.rt.workspace.get("logits", (h.shape[0], self.spec.vocab_size), torch.float32)
         self.rt.ops.gemm(h, self.weight, logits)
+        return logits
+
+
+@dataclass(frozen=True)
+class CappedHeadSpec(PartSpec):
+    """A linear head whose logits are squashed into (-cap, cap): cap * tanh(logits / cap)."""
+    kind = "capped_linear_head"
+    vocab_size: int = 0
+    hidden_size: int = 0
+    cap: float = 30.0
+
+
+@register_head(CappedHeadSpec.kind)
+class CappedLinearHead(LinearHead):
+    spec_class = CappedHeadSpec
+
+    def __init__(self, spec: CappedHeadSpec, tensors: Dict[str, torch.Tensor], rt: Runtime):
+        if not spec.cap > 0:
+            raise ValueError(f"a logit cap must be positive, got {spec.cap}")
+        super().__init__(spec, tensors, rt)
+
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        logits = super().forward(h, ctx)
+        self.rt.ops.soft_cap(logits, self.spec.cap)
         return logits
