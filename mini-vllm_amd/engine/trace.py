@@ -37,7 +37,7 @@ class TraceError(RuntimeError):
 
 class TraceRunner:
     def __init__(self, model: str, dtype: str, max_tokens: int, page_size: int = 16, use_graph: bool = True,
-                 max_live: int = 4, enable_prefix_caching: bool = False, poison_pages: bool = False):
+                 max_live: int = 16, enable_prefix_caching: bool = False, poison_pages: bool = False):
         if TOKEN_ROUNDING % page_size:
             raise ValueError(f"the page size {page_size} must divide {TOKEN_ROUNDING}")
         max_tokens = max(TOKEN_ROUNDING, -(-max_tokens // TOKEN_ROUNDING) * TOKEN_ROUNDING)

@@ -37,7 +37,9 @@ def plan_tensors(plan: ModelPlan) -> List[Tuple[TensorLocation, TensorDecl]]:
     for i, layer in enumerate(plan.layers):
         block_cls = BLOCKS.get(layer.block.kind)
         slots = dict(layer.norms)
-        for slot in getattr(block_cls, "norm_slots", tuple(slots)):
+        needed = (block_cls.slots_for(layer.ffn is not None) if hasattr(block_cls, "slots_for")
+                  else getattr(block_cls, "norm_slots", tuple(slots)))
+        for slot in needed:
             if slot not in slots:
                 raise ValueError(f"layer {i}: block arrangement {layer.block.kind!r} needs a norm for slot {slot!r}")
         for slot, nspec in layer.norms:

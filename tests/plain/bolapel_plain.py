@@ -34,10 +34,6 @@ def token_shift(h: torch.Tensor, mix: torch.Tensor, before: Optional[torch.Tenso
     return h + (prev - h) * mix
 
 
-def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def delta_rule_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, rate: torch.Tensor,
                     state: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """One head of the generalised delta rule, token by token.
@@ -58,22 +54,23 @@ def delta_rule_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: to
 
 
 def general_delta_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, heads: int, dim: int,
-                        eps: float) -> torch.Tensor:
-    """h [n, width] -> [n, width]."""
+                        eps: float, rnd=None) -> torch.Tensor:
+    """h [n, width] -> [n, width]. ``rnd`` rounds what an engine with 16-bit activations would store."""
+    rnd = rnd or (lambda t: t)
     n = h.shape[0]
     g = lambda name: w[prefix + name]
-    r = (h @ g("r").T).view(n, heads, dim)
-    k = (h @ g("k").T).view(n, heads, dim)
-    v = (h @ g("v").T).view(n, heads, dim)
-    lora = torch.tanh(h @ g("w1").T) @ g("w2").T + g("w0")
+    r = rnd(h @ g("r").T).view(n, heads, dim)
+    k = rnd(h @ g("k").T).view(n, heads, dim)
+    v = rnd(h @ g("v").T).view(n, heads, dim)
+    lora = torch.tanh(rnd(h @ g("w1").T)) @ g("w2").T + g("w0")
     decay = torch.exp(-DECAY_RATE * torch.sigmoid(lora)).view(n, heads, dim)
-    rate = torch.sigmoid(h @ g("a").T + g("a.b")).view(n, heads, dim)
+    rate = torch.sigmoid(rnd(h @ g("a").T) + g("a.b")).view(n, heads, dim)
     out = torch.empty(n, heads, dim, dtype=h.dtype)
     for j in range(heads):
         o, _ = delta_rule_scan(r[:, j], k[:, j], v[:, j], decay[:, j], rate[:, j])
         out[:, j] = rms_norm(o, None, eps)
-    y = out.reshape(n, heads * dim) * g("norm") * torch.sigmoid(h @ g("g").T)
-    return y @ g("o").T
+    y = rnd(out.reshape(n, heads * dim) * g("norm") * torch.sigmoid(rnd(h @ g("g").T)))
+    return rnd(y @ g("o").T)
 
 
 def partial_rotary(x: torch.Tensor, positions: torch.Tensor, dims: int, base: float) -> torch.Tensor:
@@ -87,19 +84,21 @@ def partial_rotary(x: torch.Tensor, positions: torch.Tensor, dims: int, base: fl
     return torch.cat((a * c - b * s, b * c + a * s, x[..., dims:]), dim=-1)
 
 
-def attention_keys_values(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, m: Dict, eps: float):
+def attention_keys_values(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, m: Dict, eps: float, rnd=None):
     """The keys (normed and rotated, as a cache would hold them) and values of a layer that owns them."""
+    rnd = rnd or (lambda t: t)
     n = h.shape[0]
-    G, D, Dv = m["kv_heads"], m["dim"], m["vdim"]
-    k = (h @ w[prefix + "k"].T).view(n, G, D)
-    v = (h @ w[prefix + "v"].T).view(n, G, Dv)
+    G, D, Dv = m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"])
+    k = rnd(h @ w[prefix + "k"].T).view(n, G, D)
+    v = rnd(h @ w[prefix + "v"].T).view(n, G, Dv)
     k = rms_norm(k, w[prefix + "k.norm"], eps)
-    k = partial_rotary(k, torch.arange(n), m["rot"]["dims"], m["rot"]["base"])
-    return k, v
+    if m.get("rot"):
+        k = partial_rotary(k, torch.arange(n), m["rot"]["dims"], m["rot"]["base"])
+    return rnd(k), v
 
 
-def chunked_sigmoid_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, bias: torch.Tensor,
-                              chunk: Optional[int]) -> torch.Tensor:
+def chunked_sigmoid_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
+                              bias: Optional[torch.Tensor], chunk: Optional[int]) -> torch.Tensor:
     """q [n, H, D], k [n, G, D], v [n, G, Dv], bias [H]. Query i sees key j <= i of its own chunk
     (i // chunk == j // chunk); the weight of a visible key is sigmoid(score + bias[h]), not
     normalised over the keys."""
@@ -112,30 +111,38 @@ def chunked_sigmoid_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     out = torch.empty(n, H, v.shape[2], dtype=q.dtype)
     for hd in range(H):
         kv = hd // (H // G)
-        score = (q[:, hd] @ k[:, kv].T) * scale + bias[hd]
+        score = (q[:, hd] @ k[:, kv].T) * scale + (0.0 if bias is None else bias[hd])
         weight = torch.sigmoid(score) * seen
         out[:, hd] = weight @ v[:, kv]
     return out
 
 
 def attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, m: Dict, eps: float,
-                    keys_values) -> torch.Tensor:
+                    keys_values, rnd=None) -> torch.Tensor:
+    rnd = rnd or (lambda t: t)
     n = h.shape[0]
     H, D = m["heads"], m["dim"]
-    q = (h @ w[prefix + "q"].T).view(n, H, D)
+    q = rnd(h @ w[prefix + "q"].T).view(n, H, D)
     q = rms_norm(q, w[prefix + "q.norm"], eps)
-    q = partial_rotary(q, torch.arange(n), m["rot"]["dims"], m["rot"]["base"])
+    if m.get("rot"):
+        q = partial_rotary(q, torch.arange(n), m["rot"]["dims"], m["rot"]["base"])
+    q = rnd(q)
     k, v = keys_values
     chunk = m["mask"]["size"] if m.get("mask") else None
     o = chunked_sigmoid_attention(q, k, v, m["scale"], w[prefix + "pb"], chunk)
-    gate = torch.sigmoid(h @ w[prefix + "g"].T)                   # [n, H]
-    o = o * gate[:, :, None]
-    return o.reshape(n, -1) @ w[prefix + "o"].T
+    gate = torch.sigmoid(rnd(h @ w[prefix + "g"].T))              # [n, H]
+    o = rnd(o * gate[:, :, None])
+    return rnd(o.reshape(n, -1) @ w[prefix + "o"].T)
 
 
-def dense_feed_forward(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str) -> torch.Tensor:
+def dense_feed_forward(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, rnd=None) -> torch.Tensor:
+    rnd = rnd or (lambda t: t)
     gate = h @ w[prefix + "gate"].T
-    return (gate * torch.sigmoid(gate) * (h @ w[prefix + "up"].T)) @ w[prefix + "down"].T
+    return rnd(rnd(gate * torch.sigmoid(gate) * (h @ w[prefix + "up"].T)) @ w[prefix + "down"].T)
+
+
+def round_to_bfloat16(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.bfloat16).to(t.dtype)
 
 
 def soft_cap(logits: torch.Tensor, cap: Optional[float]) -> torch.Tensor:
@@ -146,8 +153,10 @@ def soft_cap(logits: torch.Tensor, cap: Optional[float]) -> torch.Tensor:
 # the model
 # ---------------------------------------------------------------------------------------
 def forward(cfg: Dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtype=torch.float64,
-            return_layers: bool = False):
-    """Logits [n, vocab] of one sequence (and the residual stream after every layer)."""
+            return_layers: bool = False, rnd=None):
+    """Logits [n, vocab] of one sequence (and the residual stream after every layer). ``rnd`` rounds
+    what an engine with 16-bit activations would store (the residual stream and the recurrence stay wide)."""
+    rnd = rnd or (lambda t: t)
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     eps = float(cfg["norm"]["eps"])
     x = w["embed"][torch.tensor(tokens, dtype=torch.long)]
@@ -155,24 +164,24 @@ def forward(cfg: Dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtyp
     kept = {}
     for i, layer in enumerate(cfg["layers"]):
         p = f"l{i}."
-        h = rms_norm(x, w[p + "norm1"], eps)
-        h = token_shift(h, w[p + "shift"])
+        h = rnd(rms_norm(x, w[p + "norm1"], eps))
+        h = rnd(token_shift(h, w[p + "shift"]))
         m = layer["mixer"]
         if layer["type"] == "general_delta":
-            y = general_delta_mixer(h, w, p + "mix.", m["heads"], m["dim"], eps)
+            y = general_delta_mixer(h, w, p + "mix.", m["heads"], m["dim"], eps, rnd)
         elif layer["type"] == "attention":
             src = m.get("kv_from")
             if src is None:
-                kept[i] = attention_keys_values(h, w, p + "mix.", m, eps)
+                kept[i] = attention_keys_values(h, w, p + "mix.", m, eps, rnd)
                 src = i
-            y = attention_mixer(h, w, p + "mix.", m, eps, kept[src])
+            y = attention_mixer(h, w, p + "mix.", m, eps, kept[src], rnd)
         else:
             raise ValueError(layer["type"])
         x = x + rms_norm(y, w[p + "norm1b"], eps)
         if layer.get("mlp") is not None:
-            h = rms_norm(x, w[p + "norm2"], eps)
-            x = x + rms_norm(dense_feed_forward(h, w, p + "mlp."), w[p + "norm2b"], eps)
+            h = rnd(rms_norm(x, w[p + "norm2"], eps))
+            x = x + rms_norm(dense_feed_forward(h, w, p + "mlp.", rnd), w[p + "norm2b"], eps)
         layers.append(x)
-    h = rms_norm(x, w["final.norm"], eps)
+    h = rnd(rms_norm(x, w["final.norm"], eps))
     logits = soft_cap(h @ w["head"].T, cfg.get("logit_softcap"))
     return (logits, torch.stack(layers)) if return_layers else logits

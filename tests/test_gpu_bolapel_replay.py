@@ -1,0 +1,214 @@
+"""Bolapel in the engine against the plain model under every way of cutting the same requests:
+whole, last tokens one by one (through graphs and without), portions of changing size down to two
+tokens, mixed with other requests on so few pages and slots that they are used again; float32 and
+bfloat16; tiny configurations that differ in every size and option; and greedy generation through
+the engine's own entry point and scheduler."""
+import numpy as np
+import pytest
+import torch
+
+import trace_tools
+from bolapel_helpers import BOLA, RANKS, make_weights, plain_logits, plain_logits_bf16, random_tokens
+from helpers import TOL_F32, bf16_tolerance, rel_err, write_model_dir
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ["P", "Q", "R", "S"]
+# longer than two chunks of every layer, so that chunk edges pass inside prompts and among decoded tokens
+LENGTHS = {"P": [70, 5, 45, 21, 33, 2], "Q": [118, 40, 66, 3, 58], "R": [150, 17, 260, 49], "S": [50, 36, 77, 1]}
+PAGE = {"P": 16, "Q": 8, "R": 16, "S": 16}
+GAINS = {"sharp": 2.0, "mild": 1.0}
+
+
+class Case:
+    def __init__(self, name, tmp, kind):
+        self.name, self.kind, self.cfg, self.page = name, kind, BOLA[name], PAGE[name]
+        self.weights = make_weights(self.cfg, RANKS[name], seed=sum(map(ord, name)), qk_gain=GAINS[kind])
+        self.dir = write_model_dir(str(tmp / f"bola{name}_{kind}"), self.cfg, self.weights)
+        self.reqs = {f"r{i}": random_tokens(self.cfg, n, seed=100 + i) for i, n in enumerate(LENGTHS[name])}
+        self.want = {rid: plain_logits(self.cfg, self.weights, toks) for rid, toks in self.reqs.items()}
+        emulated = {rid: plain_logits_bf16(self.cfg, self.weights, toks) for rid, toks in self.reqs.items()}
+        self.bf16_error = max(rel_err(emulated[rid][p], self.want[rid][p])
+                              for rid, toks in self.reqs.items() for p in range(len(toks)))
+
+    def tol(self, dtype):
+        return TOL_F32 if dtype == "float32" else bf16_tolerance(self.bf16_error)
+
+    def check(self, got, dtype, what):
+        worst = max(rel_err(row, self.want[rid][pos]) for (rid, pos), row in got.items())
+        print(f"{what} [{dtype}]: {len(got)} rows, worst relative error {worst:.3e} (allowed {self.tol(dtype):.3e})")
+        assert worst <= self.tol(dtype), f"{what}: worst relative error {worst:.3e} exceeds {self.tol(dtype):.1e}"
+        return sum(len(t) for t in self.reqs.values())
+
+
+@pytest.fixture(scope="module")
+def cases(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("bolapel")
+    return {(name, kind): Case(name, tmp, kind) for name in NAMES for kind in GAINS}
+
+
+def runner_for(case, dtype, steps, page_size=None, use_graph=True, **kw):
+    from minivllm_amd.engine.trace import TraceRunner
+    return TraceRunner(case.dir, dtype, trace_tools.max_live_tokens(steps), page_size=page_size or case.page,
+                       use_graph=use_graph, **kw)
+
+
+def both(cases, name):
+    return [cases[(name, kind)] for kind in GAINS]
+
+
+def prompt_lens_of(case):
+    return {rid: max(2, len(t) - 12) if len(t) > 3 else len(t) for rid, t in case.reqs.items()}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", NAMES)
+def test_whole(cases, name, dtype):
+    for case in both(cases, name):
+        steps = trace_tools.whole(case.reqs)
+        got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
+        assert len(got) == case.check(got, dtype, f"{name} {case.kind} whole")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("use_graph", [True, False])
+def test_tail_decode(cases, name, dtype, use_graph):
+    """The last 60 tokens one by one: longer than every chunk but R's second, so chunk edges pass among them."""
+    for case in both(cases, name):
+        steps = trace_tools.tail_decode(case.reqs, tail=60)
+        got = trace_tools.collect(steps, runner_for(case, dtype, steps, use_graph=use_graph).run_step)
+        case.check(got, dtype, f"{name} {case.kind} last 60 one by one (graph={use_graph})")
+        assert all((rid, len(toks) - 1) in got for rid, toks in case.reqs.items())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("page_size", ["own", 4])
+def test_portions(cases, name, dtype, page_size):
+    for case in both(cases, name):
+        steps = trace_tools.portions(case.reqs)
+        ps = case.page if page_size == "own" else page_size
+        got = trace_tools.collect(steps, runner_for(case, dtype, steps, page_size=ps).run_step)
+        assert len(got) == case.check(got, dtype, f"{name} {case.kind} portions (page {ps})")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", NAMES)
+def test_mixed(cases, name, dtype):
+    """Up to three live requests on three state slots and pages for exactly the live tokens: slots and
+    pages change hands, and a slot's state and shift row from the request before must not leak."""
+    for case in both(cases, name):
+        for seed in (0, 1):
+            steps = trace_tools.mixed(case.reqs, prompt_lens_of(case), max_live=3, seed=seed)
+            runner = runner_for(case, dtype, steps, max_live=3)
+            got = trace_tools.collect(steps, runner.run_step)
+            assert len(got) == case.check(got, dtype, f"{name} {case.kind} mixed seed {seed}")
+            runner.manager.check_invariants()
+            assert not runner.manager.seqs and runner.manager.slots.num_free == 3
+            for pool in runner.manager.pools:
+                assert pool.num_free == pool.num_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", NAMES)
+def test_steps_with_prompt_portions_from_graphs(cases, name, dtype):
+    """Every entry wants its last row only, as generation does: such steps are replayed from graphs per
+    size class, padded with inert rows and sequences that must leave every state alone."""
+    case = cases[(name, "sharp")]
+    cuttings = {"portions": trace_tools.portions(case.reqs),
+                "mixed": trace_tools.mixed(case.reqs, prompt_lens_of(case), max_live=4, seed=4)}
+    for what, steps in cuttings.items():
+        steps = trace_tools.only_last_rows(steps)
+        runner = runner_for(case, dtype, steps)
+        got = trace_tools.collect(steps, runner.run_step)
+        case.check(got, dtype, f"{name} {what} from graphs")
+        assert len(got) == sum(len(st["entries"]) for st in steps)
+        assert runner.executor.model.graph_safe and list(runner.executor._mixed_graphs)
+        eager = trace_tools.collect(steps, runner_for(case, dtype, steps, use_graph=False).run_step)
+        worst = max(rel_err(got[k], eager[k]) for k in got)
+        assert worst <= (1e-6 if dtype == "float32" else 2e-2), f"graphs against eager steps: {worst:.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_mixed_with_poisoned_pages(cases, name, dtype):
+    """Pages are filled with NaN when they change hands, also the ones a chunk has passed: a kernel that
+    reads a slot nobody has written since, or a page that was given back, puts NaN into the logits."""
+    case = cases[(name, "sharp")]
+    steps = trace_tools.mixed(case.reqs, prompt_lens_of(case), max_live=4, seed=2)
+    runner = runner_for(case, dtype, steps, poison_pages=True)
+    got = trace_tools.collect(steps, runner.run_step)
+    assert len(got) == case.check(got, dtype, f"{name} mixed on poisoned pages")
+
+
+def test_pages_go_back_when_a_chunk_has_passed(cases):
+    case = cases[("P", "mild")]                               # chunks of 20 on pages of 4
+    from minivllm_amd.engine.trace import TraceRunner
+    runner = TraceRunner(case.dir, "float32", 128, page_size=4)
+    toks = case.reqs["r0"]
+    runner.run_step({"step": 0, "entries": [{"id": "a", "tokens": toks[:47], "want": [46]}], "end": []})
+    table = runner.manager.block_table("a", 0)
+    assert all(p < 0 for p in table[:10]) and all(p >= 0 for p in table[10:12])        # positions 40.. stay
+    out = runner.run_step({"step": 1, "entries": [{"id": "a", "tokens": toks[47:70], "want": [0, 12, 13, 22]}], "end": ["a"]})
+    for row, pos in zip(out, (47, 59, 60, 69)):
+        assert rel_err(row, case.want["r0"][pos]) <= TOL_F32
+    assert runner.manager.pools[0].num_free == runner.manager.pools[0].num_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_and_short_requests(cases, dtype):
+    case = cases[("Q", "sharp")]
+    reqs = {"one": case.reqs["r0"][:1], "two": case.reqs["r0"][:2], "three": case.reqs["r1"][:3]}
+    steps = trace_tools.whole(reqs)
+    got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
+    for (rid, pos), row in got.items():
+        assert rel_err(row, case.want["r0" if rid in ("one", "two") else "r1"][pos]) <= case.tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(cases, dtype):
+    """Four tokens of prompt, then 250 tokens one by one: many chunks and pages pass, the state runs on."""
+    case = cases[("P", "mild")]
+    toks = random_tokens(case.cfg, 254, seed=9)
+    want = plain_logits(case.cfg, case.weights, toks)
+    steps = trace_tools.tail_decode({"long": toks}, tail=250)
+    got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
+    tol = TOL_F32 if dtype == "float32" else bf16_tolerance(
+        max(rel_err(a, b) for a, b in zip(plain_logits_bf16(case.cfg, case.weights, toks), want)))
+    worst = max(rel_err(row, want[pos]) for (_, pos), row in got.items())
+    assert len(got) == 251 and worst <= tol, f"worst relative error {worst:.3e} exceeds {tol:.1e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "R"])
+def test_greedy_generation(cases, name, dtype):
+    """Through LLM.generate: the scheduler cuts prompts into portions of at most 24 tokens, batches
+    them with decoding requests, runs decode steps in rows from graphs, and preempts when pages run out."""
+    from minivllm_amd import LLM, SamplingParams
+    case = cases[(name, "mild")]
+    llm = LLM(model=case.dir, dtype=dtype, kv_cache_block_size=case.page, kv_cache_num_blocks=40, max_model_len=320,
+              max_num_batched_tokens=48, max_num_batched_seqs=4, prefill_chunk=24)
+    prompts = [random_tokens(case.cfg, n, seed=n) for n in (5, 61, 33, 1, 90, 18)]
+    sp = SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True)
+    outs = llm.generate(prompts, sp, use_tqdm=False)
+    assert [o.prompt_token_ids for o in outs] == prompts and all(len(o.token_ids) == 40 for o in outs)
+    clear = near = 0
+    for out in outs:
+        seq = list(out.prompt_token_ids) + list(out.token_ids)
+        logits = plain_logits(case.cfg, case.weights, seq)
+        tol = TOL_F32 if dtype == "float32" else bf16_tolerance(
+            max(rel_err(a, b) for a, b in zip(plain_logits_bf16(case.cfg, case.weights, seq), logits)))
+        for t, tok in enumerate(out.token_ids):
+            row = logits[len(out.prompt_token_ids) + t - 1]
+            slack = 2 * tol * float(np.abs(row).max())
+            assert row[tok] >= row.max() - slack, f"token {t}: {tok} scores {row[tok]}, the best {row.max()}"
+            if row.max() - np.partition(row, -2)[-2] > slack:
+                assert tok == int(row.argmax())
+                clear += 1
+            else:
+                near += 1
+    print(f"greedy {name} [{dtype}]: {clear} tokens decided by a clear margin, {near} near ties")
+    # (random weights give flat logits: in bfloat16 most choices are near ties, which only have to lie within the slack)
+    assert clear > near if dtype == "float32" else clear >= 20
+    llm.manager.check_invariants()
