@@ -73,8 +73,12 @@ def build_llm(args, shape, layers, max_seqs=None, token_budget=None, num_pages=N
     from minivllm_amd.models import config_from_dict, expected_tensors
     from minivllm_amd.weights.device_random import DeviceRandomSource
 
-    raw = dict(shape, architectures=["Qwen3ForCausalLM"], num_hidden_layers=layers,
-               max_position_embeddings=40960, torch_dtype=args.dtype)
+    if getattr(args, "design", "qwen3") == "bolapel":
+        from minivllm_amd.config.shapes import bolapel_shape
+        raw = dict(bolapel_shape(args.shape, layers, chunk=args.chunk), torch_dtype=args.dtype)
+    else:
+        raw = dict(shape, architectures=["Qwen3ForCausalLM"], num_hidden_layers=layers,
+                   max_position_embeddings=40960, torch_dtype=args.dtype)
     arch, cfg = config_from_dict(raw)
     dev = torch.device("cuda:0")
     stored = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
@@ -254,7 +258,7 @@ def emit_kernels(llm, cfg, args) -> int:
         key = max(rows, key=lambda t: (-t[0], t[2])) if rows else min(single)
         ledger = roofline.one_step(roofline.launches(ex.graph_ledger[key]))
         ctx = args.prompt_len + (args.warmup + args.steps) // 2
-        title = (f"decode step, qwen3-{args.shape} shape, batch {args.batch}, priced at a context of {ctx} tokens "
+        title = (f"decode step, {args.design}-{args.shape} shape, batch {args.batch}, priced at a context of {ctx} tokens "
                  f"(graph for {key[0]} sequences, contexts up to {key[1]})")
         print(roofline.kernel_table(args.emit_kernels, ledger, args.dtype, keys=args.batch * ctx, pairs=args.batch * ctx,
                                     title=title, wall_ms=args.step_ms))
@@ -274,9 +278,81 @@ def emit_kernels(llm, cfg, args) -> int:
             ledger = roofline.launches(lines)
         finally:
             ex.ops.ledger = None
-        title = f"prefill of one {args.prefill_tokens}-token prompt, qwen3-{args.shape} shape"
+        title = f"prefill of one {args.prefill_tokens}-token prompt, {args.design}-{args.shape} shape"
         print(roofline.kernel_table(args.emit_kernels, ledger, args.dtype, title=title,
                                     wall_ms=args.step_ms if args.only == "prefill" else None))
+    return 0
+
+
+def bolapel_numbers(llm, cfg, item):
+    """From the loaded model: elements of all tensors, of the matrices the step multiplies with, bytes of
+    state a request reads and writes a step, cache bytes a token takes, and per attention layer
+    (heads, key size, value size, chunk)."""
+    from minivllm_amd.models.causal_lm import expected_tensors
+    ex = llm.executor
+    decls = expected_tensors(ex.arch, cfg, ex.plan)
+    params = sum(_numel(d.shape) for d in decls.values())
+    matrices = sum(_numel(d.shape) for n, d in decls.items() if len(d.shape) == 2 and n != "embed")
+    state_bytes = sum(t[0].numel() * t.element_size() for ts in ex.state_tensors.values() for t in ts.values())
+    kv_bytes = sum(need.bytes_per_token(ex.dtype) for need in ex.needs if need is not None)
+    attn = [(l.heads, l.dim, l.vdim, l.chunk) for l in cfg.layers if l.type == "attention"]
+    delta = [(l.heads, l.dim) for l in cfg.layers if l.type == "general_delta"]
+    return dict(params=params, matrices=matrices, state_bytes=state_bytes, kv_bytes=kv_bytes, attn=attn, delta=delta)
+
+
+def _numel(shape):
+    n = 1
+    for d in shape:
+        n *= int(d)
+    return n
+
+
+def bench_bolapel(args, llm, cfg, layers, layers_full, item) -> int:
+    """The default measurements for a Bolapel model of the named shape; the same fields in the line."""
+    nums = bolapel_numbers(llm, cfg, item)
+    prefill = None
+    if args.only in ("all", "prefill"):
+        prefill_s = measure_prefill(llm, cfg.vocab_size, args.prefill_tokens, repeats=3, seed=args.seed)
+        T = args.prefill_tokens
+        flops = 2 * T * (nums["matrices"] - cfg.vocab_size * cfg.hidden_size) + 2 * cfg.vocab_size * cfg.hidden_size
+        for H, D, Dv, chunk in nums["attn"]:
+            c = min(chunk or T, T)
+            flops += 2 * H * (D + Dv) * (T // c) * c * (c + 1) // 2 * 1 + 2 * H * (D + Dv) * (T % c) * (T % c + 1) // 2
+        for H, D in nums["delta"]:
+            flops += 8 * T * H * D * D                     # four multiply-adds per state element and token
+        prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+                   "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+    tok_s = ms_step = roofline = None
+    ran = regions = 0
+    if args.only in ("all", "decode"):
+        tok_s, ms_step, mean_ctx, ran, regions = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len,
+                                                                args.steps, args.warmup, args.seed)
+        # every weight once, each request's states read and written, the keys and values of its current chunk
+        seen = sum(min(chunk or mean_ctx, mean_ctx) / 2.0 if chunk else mean_ctx for _, _, _, chunk in nums["attn"]) \
+            / max(1, len(nums["attn"]))
+        step_bytes = nums["params"] * item + args.batch * (2 * nums["state_bytes"] + seen * nums["kv_bytes"])
+        achieved = step_bytes / (ms_step * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(achieved / PEAK_HBM_GBS, 4)}
+    points = {}
+    if not args.no_points and args.only == "all":
+        for b, key in ((1, "decode_b1"), (64, "decode_b64")):
+            n = min(args.steps, 128)
+            points[key] = round(measure_decode(llm, cfg.vocab_size, b, args.prompt_len, n, min(args.warmup, 8),
+                                               args.seed + b)[0], 1)
+    config = {"model": f"bolapel-{args.shape}-shape-random", "layers": layers, "layers_full": layers_full,
+              "hidden": cfg.hidden_size, "vocab": cfg.vocab_size, "attention_layers": len(nums["attn"]),
+              "delta_layers": len(nums["delta"]), "chunk": args.chunk, "global_batch": args.batch, "seq_len": args.context,
+              "prompt_len": args.prompt_len, "block_size": args.block_size, "graph": not args.no_graph,
+              "scheduler_steps": args.scheduler_steps, "launch_ahead": bool(llm.config.launch_ahead),
+              "parallelism": "single-gpu"}
+    print(json.dumps({"metric": "decode tok/s (batch %d, %d-token prompts)" % (args.batch, args.prompt_len),
+                      "value": round(tok_s, 1) if tok_s is not None else None, "unit": "tokens/s", "n_gpus": 1,
+                      "steps": ran if ran else args.steps, "warmup": args.warmup,
+                      "ms_per_step": round(ms_step, 4) if ms_step is not None else None, "higher_is_better": True,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                      "data": "synthetic", "config": config, "timed_regions": regions, "prefill": prefill,
+                      "roofline": roofline, "points": points}))
     return 0
 
 
@@ -286,6 +362,11 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--shape", choices=sorted(SHAPES), default="0.6b")
+    ap.add_argument("--design", choices=["qwen3", "bolapel"], default="qwen3",
+                    help="'bolapel': the same widths, head counts, vocabulary and number of layers as the named Qwen3 "
+                         "shape, as a Bolapel model (three delta-rule layers to one attention layer in chunks of --chunk "
+                         "tokens); decode and prefill are measured the same way and the line names the design")
+    ap.add_argument("--chunk", type=int, default=1024, help="--design bolapel: tokens in a chunk of its attention layers")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in the record)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=1024)
@@ -379,8 +460,10 @@ def main() -> int:
     llm, cfg = build_llm(args, shape, layers)
     if args.emit_kernels:
         return emit_kernels(llm, cfg, args)
-    nums = model_numbers(shape, layers)
     item = 2 if args.dtype == "bfloat16" else 4
+    if args.design == "bolapel":
+        return bench_bolapel(args, llm, cfg, layers, layers_full, item)
+    nums = model_numbers(shape, layers)
 
     prefill = None
     if args.only in ("all", "prefill"):

@@ -42,3 +42,31 @@ def qwen3_shape(name: str, **overrides) -> Dict[str, Any]:
     raw = dict(QWEN3_SHAPES[name], architectures=["Qwen3ForCausalLM"], max_position_embeddings=40960)
     raw.update(overrides)
     return raw
+
+
+def bolapel_shape(name: str, layers: int = None, chunk: int = 1024, delta_head_dim: int = 64, decay_rank: int = 64,
+                  pattern: int = 4) -> Dict[str, Any]:
+    """A Bolapel configuration with the width, feed-forward, vocabulary, head counts and head size of
+    the named Qwen3 shape and as many layers: every ``pattern``-th layer is attention in chunks of
+    ``chunk`` tokens (rotation over half of each head; every second of them reads the keys and values
+    of the one before), the others are delta-rule layers with heads of ``delta_head_dim``. For
+    random-weights models at sizes that resemble a real model's layers."""
+    q = QWEN3_SHAPES[name]
+    n = layers or q["num_hidden_layers"]
+    hid, hd = q["hidden_size"], q["head_dim"]
+    ff = {"kind": "dense", "ff": q["intermediate_size"]}
+    out, owner = [], None
+    for i in range(n):
+        if i % pattern == pattern - 1:
+            m = {"heads": q["num_attention_heads"], "kv_heads": q["num_key_value_heads"], "dim": hd, "vdim": hd,
+                 "scale": hd ** -0.5, "mask": {"size": chunk}, "rot": {"dims": hd // 2, "base": q["rope_theta"]}}
+            if owner is not None:
+                m["kv_from"], owner = owner, None
+            else:
+                owner = i
+            out.append({"type": "attention", "mixer": m, "mlp": ff})
+        else:
+            out.append({"type": "general_delta", "mlp": ff,
+                        "mixer": {"heads": hid // delta_head_dim, "dim": delta_head_dim, "rank": decay_rank}})
+    return {"architecture": "Bolapel", "vocab": q["vocab_size"], "width": hid, "layers": out,
+            "norm": {"eps": q["rms_norm_eps"]}, "logit_softcap": 30.0}

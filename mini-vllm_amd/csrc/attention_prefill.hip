@@ -58,13 +58,27 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // Two workgroups share a compute unit (LDS and latency hiding are sized for that), so a wave may
 // use half of a SIMD's registers: the accumulators stay in the vector registers and the operand
 // reads from LDS run ahead of the MFMAs.
-template <int D, int NT, int KW>
+//
+// SIG: sigmoid weights instead of the softmax. The weight of a visible key is
+// sigmoid(score * scale + bias[head]); nothing is normalised over the keys, so there is no running
+// maximum and no sum, and a masked score (-inf) gives the weight 0 by itself. A column's keys start at
+// max(start of its chunk, position - window, 0), chunks being runs of `chunk` positions counted from
+// the sequence's start (chunk <= 0: none). At the end head h's row is multiplied by
+// sigmoid(gate[token][h]) when gates are given.
+struct SigmoidArgs {
+    int chunk;
+    const float* bias;         // [H] or null
+    const bf16* gate;          // rows of at least H values, or null
+    long gate_stride;
+};
+
+template <int D, int NT, int KW, bool SIG = false>
 __global__ void __launch_bounds__(AP_THREADS * KW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                          const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                          const int* __restrict__ block_table, int bt_width, int page_size, int page_shift,
                          const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs, int H,
-                         int Hkv, float scale, int window, int fold) {
+                         int Hkv, float scale, int window, int fold, SigmoidArgs sig) {
     constexpr int DS = D / 32;                 // k-steps of the score product
     constexpr int DT = D / 16;                 // d tiles of the output product
     constexpr int COLS = 16 * AP_WAVES * NT;   // columns of a workgroup
@@ -137,6 +151,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     // ---- this lane's columns
     int col_tok[NT], col_head[NT], col_pos[NT], col_lo[NT];
     bool col_ok[NT];
+    float col_bias[NT];         // SIG: the head's score bias, in the base-2 domain
     Frag qop[NT][DS];
     int hi_w = -1, lo_w = 0x7fffffff;
 #pragma unroll
@@ -147,6 +162,14 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         col_head[ct] = kvh * G + (col_ok[ct] ? col % G : 0);
         col_pos[ct] = col_ok[ct] ? positions[col_tok[ct]] : -1;
         col_lo[ct] = (window >= 0 && col_pos[ct] - window > 0) ? col_pos[ct] - window : 0;
+        col_bias[ct] = 0.f;
+        if constexpr (SIG) {
+            if (sig.chunk > 0 && col_pos[ct] >= 0) {
+                const int c0 = col_pos[ct] / sig.chunk * sig.chunk;
+                col_lo[ct] = c0 > col_lo[ct] ? c0 : col_lo[ct];
+            }
+            if (sig.bias != nullptr) col_bias[ct] = sig.bias[col_head[ct]] * LOG2E;
+        }
         if (col_ok[ct]) {
             hi_w = col_pos[ct] > hi_w ? col_pos[ct] : hi_w;
             lo_w = col_lo[ct] < lo_w ? col_lo[ct] : lo_w;
@@ -281,7 +304,8 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     auto mend = [&](int j, bool gone, uint4* stage) {
         const int b = block_of(j);
         const bool tail = 32 * b + 31 > hi_g;
-        if (!tail && !(window >= 0 && __any(gone))) return;
+        const bool gives_back = window >= 0 || (SIG && sig.chunk > 0);   // pages below every column's range may be gone
+        if (!tail && !(gives_back && __any(gone))) return;
         uint4* sV = stage + kg * TILE + KCHUNKS;
 #pragma unroll
         for (int rep = 0; rep < VREP; ++rep) {
@@ -390,6 +414,18 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         }
         // online softmax per column
         Frag pop[NT];
+        if constexpr (SIG) {
+#pragma unroll
+            for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        // 1 / (1 + 2^-x); a masked score is -inf: 2^inf = inf, 1 / inf = 0
+                        const float x = fmaf(p[ct][t][r], sc_mul, col_bias[ct]);
+                        pop[ct].v[t * 4 + r] = (__bf16)__builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-x));
+                    }
+        } else
 #pragma unroll
         for (int ct = 0; ct < NT; ++ct) {
             float mx = -INFINITY;
@@ -588,8 +624,9 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
                 if (kg == 0) {
                     const float m1 = xm[cw * 16 + i], l1 = xl[cw * 16 + i];
                     const float m_fin = fmaxf(m_run[ct], m1);
-                    const float f0 = (m_run[ct] == -INFINITY) ? 0.f : exp2f(m_run[ct] - m_fin);
-                    const float f1 = (m1 == -INFINITY) ? 0.f : exp2f(m1 - m_fin);
+                    // (sigmoid weights are plain sums: the two halves just add)
+                    const float f0 = SIG ? 1.f : ((m_run[ct] == -INFINITY) ? 0.f : exp2f(m_run[ct] - m_fin));
+                    const float f1 = SIG ? 1.f : ((m1 == -INFINITY) ? 0.f : exp2f(m1 - m_fin));
                     m_run[ct] = m_fin;
                     l_run[ct] = f0 * l_run[ct] + f1 * l1;
 #pragma unroll
@@ -606,7 +643,16 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
 #pragma unroll
     for (int ct = 0; ct < NT; ++ct) {
         if (!col_ok[ct]) continue;
-        const float inv = 1.f / l_run[ct];
+        float inv;
+        if constexpr (SIG) {
+            inv = 1.f;
+            if (sig.gate != nullptr) {
+                const float z = to_f(sig.gate[(size_t)col_tok[ct] * sig.gate_stride + col_head[ct]]);
+                inv = 1.f / (1.f + __expf(-z));
+            }
+        } else {
+            inv = 1.f / l_run[ct];
+        }
         bf16* orow = out + (size_t)col_tok[ct] * out_stride + (size_t)col_head[ct] * D;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -624,15 +670,15 @@ extern "C" int mv_attention_prefill_unit_tokens(int group, int nt) {
     return group > 0 && group <= cols ? cols / group : 0;
 }
 
-template <int D, int NT, int KW>
+template <int D, int NT, int KW, bool SIG = false>
 static int launch_prefill(dim3 grid, hipStream_t stream, const void* q, long q_stride, void* out, long out_stride,
                           const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
                           int page_size, int page_shift, const int* positions, const int* cu_seqlens, int n_seqs,
-                          int H, int Hkv, float scale, int window, int fold) {
+                          int H, int Hkv, float scale, int window, int fold, SigmoidArgs sig = SigmoidArgs{0, nullptr, nullptr, 0}) {
     // the stages of K and V tiles are static LDS (four of 16 KiB per key group with D = 128)
-    hipLaunchKernelGGL((attention_prefill_kernel<D, NT, KW>), grid, dim3(AP_THREADS * KW), 0, stream, (const bf16*)q,
+    hipLaunchKernelGGL((attention_prefill_kernel<D, NT, KW, SIG>), grid, dim3(AP_THREADS * KW), 0, stream, (const bf16*)q,
                        q_stride, (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table,
-                       bt_width, page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, fold);
+                       bt_width, page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, fold, sig);
     return 0;
 }
 
@@ -687,4 +733,57 @@ extern "C" int mv_attention_prefill(const void* q, long q_stride, void* out, lon
 #undef AP_LAUNCH
     if (rc) return rc;
     return mv_check_launch("attention_prefill");
+}
+
+// The same walk with sigmoid weights (see SIG above): keys and values of one size, 64 or 128. Arguments as
+// mv_attention_prefill, then the chunk (<= 0: none), the per-head score bias (float [H] or null) and the
+// per-head gates (rows of the activation type with at least H values, or null).
+extern "C" int mv_attention_prefill_sigmoid(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
+                                            const void* v_pages, const int* block_table, int bt_width, int page_size,
+                                            const int* positions, const int* cu_seqlens, int n_seqs, int n_units,
+                                            int n_busy, int nt, int kw, int H, int Hkv, int D, float scale, int window,
+                                            int chunk, const float* bias, const void* gate, long gate_stride,
+                                            hipStream_t stream) {
+    MV_REQUIRE(kw == 1 || kw == 2, "attention_prefill_sigmoid: %d key groups per workgroup (1 or 2)", kw);
+    MV_REQUIRE(H > 0 && Hkv > 0 && H % Hkv == 0, "attention_prefill_sigmoid: %d heads are not a multiple of %d kv heads",
+               H, Hkv);
+    MV_REQUIRE(D == 64 || D == 128, "attention_prefill_sigmoid: head size %d is not served by the MFMA kernel (64 or 128)", D);
+    MV_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0,
+               "attention_prefill_sigmoid: page size %d must be a power of two, at least 16", page_size);
+    MV_REQUIRE(bt_width > 0, "attention_prefill_sigmoid: empty block table");
+    MV_REQUIRE(q_stride >= (long)H * D && q_stride % 8 == 0 && out_stride >= (long)H * D && out_stride % 4 == 0,
+               "attention_prefill_sigmoid: row strides %ld / %ld do not fit %d heads of %d", q_stride, out_stride, H, D);
+    MV_REQUIRE(gate == nullptr || gate_stride >= H, "attention_prefill_sigmoid: gate rows too short");
+    MV_REQUIRE(n_units <= 65535, "attention_prefill_sigmoid: %d units exceed one launch", n_units);
+    MV_REQUIRE(mv_attention_prefill_unit_tokens(H / Hkv, nt) > 0, "attention_prefill_sigmoid: %d query heads per kv head "
+               "with %d column tiles per wave are not served", H / Hkv, nt);
+    if (n_seqs <= 0 || n_units <= 0) return 0;
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    dim3 grid(Hkv, n_units, 1);
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        cus = 256;
+    if (n_busy <= 0 || n_busy > n_units) n_busy = n_units;
+    const int fold = (kw == 1 && (long)Hkv * n_busy <= 2L * cus) ? 1 : 0;
+    const SigmoidArgs sig{chunk, bias, (const bf16*)gate, gate_stride};
+    int rc = 0;
+#define AP_LAUNCH(DD, NN, KK)                                                                                          \
+    rc = launch_prefill<DD, NN, KK, true>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table,     \
+                                          bt_width, page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale, \
+                                          window, fold, sig)
+    if (kw == 2) {
+        if (D == 128 && nt == 2) AP_LAUNCH(128, 2, 2);
+        else if (D == 128) AP_LAUNCH(128, 1, 2);
+        else if (nt == 2) AP_LAUNCH(64, 2, 2);
+        else AP_LAUNCH(64, 1, 2);
+    } else {
+        if (D == 128 && nt == 2) AP_LAUNCH(128, 2, 1);
+        else if (D == 128) AP_LAUNCH(128, 1, 1);
+        else if (nt == 2) AP_LAUNCH(64, 2, 1);
+        else AP_LAUNCH(64, 1, 1);
+    }
+#undef AP_LAUNCH
+    if (rc) return rc;
+    return mv_check_launch("attention_prefill_sigmoid");
 }

@@ -134,6 +134,10 @@ _OPTIONAL_SIGNATURES = {
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_float, c_int, c_void_p]),
     "mv_attention_prefill_unit_tokens": (c_int, [c_int, c_int]),
+    # as mv_attention_prefill up to window, then chunk, bias, gate, gate_stride, stream
+    "mv_attention_prefill_sigmoid": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                             c_float, c_int, c_int, c_void_p, c_void_p, c_long, c_void_p]),
     "mv_launch_empty": (c_int, [c_int, c_int, c_void_p, c_void_p]),
 }
 

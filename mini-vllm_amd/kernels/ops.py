@@ -611,7 +611,20 @@ class Ops:
         w = -1 if window is None else int(window)
         qs = q.stride(0) if n > 1 else q.shape[1]
         os_ = out.stride(0) if n > 1 else num_heads * value_dim
-        self._note("mv_attention_sigmoid", self._size(q, out), 0)
+        group = num_heads // num_kv_heads
+        if (self.use_fast_kernels and plan is not None and self.lib.has("mv_attention_prefill_sigmoid")
+                and head_dim == value_dim and head_dim in (64, 128) and page_size >= 16 and not page_size & (page_size - 1)
+                and qs % 8 == 0 and os_ % 4 == 0 and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0):
+            nt, kw, n_units, n_busy = self._prefill_variant(plan, group, num_kv_heads)
+            if nt:
+                self._note_attention("mv_attention_prefill_sigmoid", plan, n, num_heads, num_kv_heads, head_dim, 2)
+                self.lib.call("mv_attention_prefill_sigmoid", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
+                              v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
+                              positions.data_ptr(), plan.cu_seqlens.data_ptr(), plan.n_seqs, n_units, n_busy, nt, kw,
+                              num_heads, num_kv_heads, head_dim, float(scale), w, c, _ptr(bias), _ptr(gate), gate_stride,
+                              self._stream())
+                return
+        self._note_attention("mv_attention_sigmoid_ref", plan, n, num_heads, num_kv_heads, head_dim, q.element_size())
         self.lib.call("mv_attention_sigmoid_ref", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size, positions.data_ptr(),
                       token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim, value_dim, float(scale), c, w,
@@ -1235,6 +1248,41 @@ class Ops:
                       DECODE_ATTENTION_WAVES, token_seq.data_ptr(), self._stream())
         return True
 
+    def _prefill_variant(self, plan, group: int, Hkv: int):
+        """(column tiles per wave, key groups per workgroup, units, busy units) of the MFMA prompt
+        attention for this step; column tiles 0: the kernel does not serve ``group`` heads per kv head."""
+        # 128 columns per workgroup (each operand read from LDS feeds two MFMAs) when that still leaves
+        # two workgroups for every compute unit, else 64 (measured on MI355X: 2048 tokens of one
+        # sequence with 8 kv heads are faster with 64, 4096 tokens or 8 x 512 with 128)
+        nt, n_units, n_busy = 0, 0, 0
+        for cand in (2, 1):
+            u = self.lib.dll.mv_attention_prefill_unit_tokens(group, cand)
+            if u > 0:
+                units, busy = plan.units(u), plan.busy_units(u)
+                if cand == 2 and busy * Hkv < 2 * self.compute_units and \
+                        self.lib.dll.mv_attention_prefill_unit_tokens(group, 1) > 0:
+                    continue
+                nt, n_units, n_busy = cand, units, busy
+                break
+        if plan.prefill_variant is not None:
+            nt = int(plan.prefill_variant[0])
+            u = self.lib.dll.mv_attention_prefill_unit_tokens(group, nt)
+            if u <= 0:
+                raise KernelLibraryError(f"attention: {nt} column tiles a wave do not serve {group} heads per kv head")
+            n_units, n_busy = plan.units(u), plan.busy_units(u)
+        if nt == 0:
+            return 0, 0, 0, 0
+        # two key groups per workgroup (eight waves) halve the walk over long contexts; they pay while
+        # the grid leaves compute units waiting for the longest walk (measured on MI355X, 8 kv heads:
+        # faster below two four-wave workgroups per compute unit, 33.9 against 35.3 us at 1,792 tokens,
+        # slower from there on, 44.0 against 40.8 us at 2,048)
+        # (a recorded step's grid is sized for the most units its size class can have; the rule goes by
+        # the units its tokens fill, as an eager step's does)
+        kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_busy * Hkv < 2 * self.compute_units else 1
+        if plan.prefill_variant is not None:
+            kw = int(plan.prefill_variant[1])
+        return nt, kw, n_units, n_busy
+
     def _attention_fast(self, q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions, token_seq,
                         H, Hkv, D, scale, window, plan) -> bool:
         """The MFMA kernels, when the step and the sizes allow them."""
@@ -1256,36 +1304,9 @@ class Ops:
             return True
         if page_size & (page_size - 1):
             return False
-        # 128 columns per workgroup (each operand read from LDS feeds two MFMAs) when that still leaves
-        # two workgroups for every compute unit, else 64 (measured on MI355X: 2048 tokens of one
-        # sequence with 8 kv heads are faster with 64, 4096 tokens or 8 x 512 with 128)
-        nt, n_units, n_busy = 0, 0, 0
-        for cand in (2, 1):
-            u = self.lib.dll.mv_attention_prefill_unit_tokens(group, cand)
-            if u > 0:
-                units, busy = plan.units(u), plan.busy_units(u)
-                if cand == 2 and busy * Hkv < 2 * self.compute_units and \
-                        self.lib.dll.mv_attention_prefill_unit_tokens(group, 1) > 0:
-                    continue
-                nt, n_units, n_busy = cand, units, busy
-                break
-        if plan.prefill_variant is not None:
-            nt = int(plan.prefill_variant[0])
-            u = self.lib.dll.mv_attention_prefill_unit_tokens(group, nt)
-            if u <= 0:
-                raise KernelLibraryError(f"attention: {nt} column tiles a wave do not serve {group} heads per kv head")
-            n_units, n_busy = plan.units(u), plan.busy_units(u)
+        nt, kw, n_units, n_busy = self._prefill_variant(plan, group, Hkv)
         if nt == 0:
             return False
-        # two key groups per workgroup (eight waves) halve the walk over long contexts; they pay while
-        # the grid leaves compute units waiting for the longest walk (measured on MI355X, 8 kv heads:
-        # faster below two four-wave workgroups per compute unit, 33.9 against 35.3 us at 1,792 tokens,
-        # slower from there on, 44.0 against 40.8 us at 2,048)
-        # (a recorded step's grid is sized for the most units its size class can have; the rule goes by
-        # the units its tokens fill, as an eager step's does)
-        kw = 2 if plan.max_context_len >= PREFILL_TWO_GROUPS_FROM and n_busy * Hkv < 2 * self.compute_units else 1
-        if plan.prefill_variant is not None:
-            kw = int(plan.prefill_variant[1])
         self._note_attention("mv_attention_prefill", plan, q.shape[0], H, Hkv, D, 2)
         self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,

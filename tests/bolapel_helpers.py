@@ -39,8 +39,9 @@ BOLA_Q = {"architecture": "Bolapel", "vocab": 333, "width": 96, "norm": {"eps": 
                      _attn(6, 1, 64, 40, 50, 32, 70000.0, 0.11, 72, kv_from=2)]}
 # R: sizes the bfloat16 serving kernels take (head size 64 for the delta rule, 128 / 64 for attention)
 BOLA_R = {"architecture": "Bolapel", "vocab": 512, "width": 256, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
-          "layers": [_delta(4, 64, 512), _attn(8, 2, 128, 64, 48, 64, 1000000.0, 0.0884, 512),
-                     _delta(2, 128, 256), _attn(8, 2, 128, 64, 112, 64, 1000000.0, 0.07, 512, kv_from=1)]}
+          "layers": [_delta(4, 64, 512), _attn(8, 2, 128, 128, 48, 64, 1000000.0, 0.0884, 512),
+                     _delta(2, 128, 256), _attn(8, 2, 128, 128, 112, 64, 1000000.0, 0.07, 512, kv_from=1),
+                     _attn(4, 4, 64, 64, 200, 64, 10000.0, 0.125, None)]}
 # S: no mask (all keys), no rotation, values as large as keys, every head its own keys
 BOLA_S = {"architecture": "Bolapel", "vocab": 150, "width": 48, "norm": {"eps": 2e-5}, "logit_softcap": 5.0,
           "layers": [_attn(2, 2, 24, 24, None, 0, 0.0, 0.2, 64), _delta(2, 12, None)]}

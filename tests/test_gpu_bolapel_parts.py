@@ -193,8 +193,15 @@ def paged(k, v, page_size, n_pages, seed):
     return kp.to(DEV), vp.to(DEV), [int(i) for i in ids]
 
 
-def run_attention(ops, q, k, v, positions, scale, chunk, window, bias, gate, page_size=4, seed=0):
+def run_attention(ops, q, k, v, positions, scale, chunk, window, bias, gate, page_size=4, seed=0, with_plan=False):
+    """``with_plan``: the step is described to the kernels' front end as the engine does (one request of
+    these rows, in row 1 of the block table), which lets it pick the MFMA kernel where the sizes allow."""
+    from minivllm_amd.engine.step import AttentionPlan
     n_q, H, D = q.shape
+    plan = None
+    if with_plan:
+        plan = AttentionPlan(decode_only=n_q == 1, max_q_len=n_q, max_context_len=max(positions) + 1, n_seqs=2,
+                             q_lens=[0, n_q], cu_seqlens=i32([0, 0, n_q]))
     Dv = v.shape[2]
     kp, vp, ids = paged(k, v, page_size, 2 * (-(-k.shape[0] // page_size)) + 3, seed)
     table = torch.full((2, len(ids) + 2), -1, dtype=torch.int32)
@@ -202,7 +209,7 @@ def run_attention(ops, q, k, v, positions, scale, chunk, window, bias, gate, pag
     out = torch.empty(n_q, H * Dv, dtype=q.dtype, device=DEV)
     ops.attention_sigmoid(q.reshape(n_q, H * D).to(DEV), out, kp, vp, table.to(DEV), page_size, i32(positions),
                           i32([1] * n_q), H, k.shape[1], D, Dv, scale, chunk, window,
-                          None if bias is None else bias.float().to(DEV), None if gate is None else gate.to(DEV))
+                          None if bias is None else bias.float().to(DEV), None if gate is None else gate.to(DEV), plan=plan)
     torch.cuda.synchronize()
     return out.view(n_q, H, Dv)
 
@@ -223,12 +230,17 @@ def test_sigmoid_attention_over_pages(dtype, H, G, D, Dv, chunk, page):
     scale = 1.7 / math.sqrt(D)
     want = plain.chunked_sigmoid_attention(q.double(), k.double(), v.double(), scale, bias.double(), chunk)
     want = want * torch.sigmoid(gate[:, :H].double())[:, :, None]
-    got = run_attention(ops, q, k, v, list(range(n)), scale, chunk, None, bias, gate, page_size=page)
-    close(got, want, 1e-5 if dtype == torch.float32 else 8e-3, "every position of a prompt")
+    for with_plan in (False, True):
+        got = run_attention(ops, q, k, v, list(range(n)), scale, chunk, None, bias, gate, page_size=page, with_plan=with_plan)
+        close(got, want, 1e-5 if dtype == torch.float32 else 8e-3, f"every position of a prompt (plan={with_plan})")
+    # a portion from the middle of the sequence, cut inside a chunk and a page
+    got = run_attention(ops, q[37:101], k[:101], v[:101], list(range(37, 101)), scale, chunk, None, bias, gate[37:101],
+                        page_size=page, with_plan=True)
+    close(got, want[37:101], 1e-5 if dtype == torch.float32 else 8e-3, "a portion")
     # single decoded tokens: the same rows, asked for one position at a time
     for p in sorted({0, 1, n - 1} | ({chunk - 1, chunk, chunk + 1, 2 * chunk - 1, 2 * chunk} if chunk and 2 * chunk < n else set())):
         one = run_attention(ops, q[p:p + 1], k[:p + 1], v[:p + 1], [p], scale, chunk, None, bias, gate[p:p + 1],
-                            page_size=page, seed=p)
+                            page_size=page, seed=p, with_plan=bool(p % 2))
         close(one, want[p:p + 1], 1e-5 if dtype == torch.float32 else 8e-3, f"position {p} alone")
 
 
@@ -248,6 +260,33 @@ def test_sigmoid_attention_sees_exactly_its_keys(dtype, chunk, window, page):
         want = torch.zeros(n)
         want[lo:i + 1] = 0.5
         assert torch.equal(got[i, 0], want) and torch.equal(got[i, 1], want), f"query {i} (keys {lo}..{i})"
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("chunk, window, page", [(10, None, 16), (64, None, 16), (None, 9, 32), (40, 13, 16), (None, None, 16),
+                                                 (100, None, 64)])
+def test_mfma_sigmoid_attention_sees_exactly_its_keys(D, chunk, window, page):
+    """The same through the MFMA kernel (bfloat16, head sizes 64 and 128, values as large as keys): the
+    value of key j is the unit vector j % D scaled by 1 + j // D, so a row still names its keys."""
+    dtype = torch.bfloat16
+    ops = ops_for(dtype)
+    n = 3 * D
+    q = torch.zeros(n, 4, D, dtype=dtype)
+    k = torch.randn(n, 2, D).to(dtype)
+    v = torch.zeros(n, 2, D)
+    for j in range(n):
+        v[j, :, j % D] = 1 + j // D
+    for rows in (range(n), range(D + 5, n - 3)):
+        rows = list(rows)
+        got = run_attention(ops, q[rows], k[:rows[-1] + 1], v[:rows[-1] + 1].to(dtype), rows, 1.0, chunk, window,
+                            torch.zeros(4), None, page_size=page, with_plan=True).float().cpu()
+        for at, i in enumerate(rows):
+            lo = max(0 if chunk is None else i // chunk * chunk, 0 if window is None else i - window)
+            want = torch.zeros(D)
+            for j in range(lo, i + 1):
+                want[j % D] += 0.5 * (1 + j // D)
+            for hd in range(4):
+                assert torch.equal(got[at, hd], want), f"query {i} head {hd} (keys {lo}..{i})"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
