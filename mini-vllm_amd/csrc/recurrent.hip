@@ -67,11 +67,14 @@ extern "C" int mv_token_shift(const void* h, long ldh, void* out, long ldo, cons
 
 // ---------------------------------------------------------------------------------------
 // Delta rule, prepare. The packed rows hold [r | k | v | g | a | w1] (H*D columns each, `rank` for
-// w1) from column 0 on. For DP_TOKENS rows and 256 channels a workgroup:
-//   coef[0][t][c] = exp(-decay_rate * sigmoid(w0[c] + sum_j W2[c][j] tanh(w1[t][j])))
-//   coef[2][t][c] = u = k[t][c] / sqrt(sum over the head of k^2 + key_eps)
-//   coef[1][t][c] = sigmoid(a[t][c] + a_bias[c]) * u
-// A row of W2 is read once for the workgroup's rows.
+// w1) from column 0 on. For DP_TOKENS rows and 256 channels a workgroup, with c = (head, d):
+//   coef[t][head][0][d] = w  = exp(-decay_rate * sigmoid(w0[c] + sum_j W2t[j][c] tanh(w1[t][j])))
+//   coef[t][head][2][d] = u  = k[t][c] / sqrt(sum over the head of k^2 + key_eps)
+//   coef[t][head][1][d] = a u, a = sigmoid(a[t][c] + a_bias[c])
+//   coef[t][head][3][d] = k[t][c],  coef[t][head][4][d] = r[t][c]                (as floats)
+// W2 comes transposed, [rank][H*D], so that neighbouring channels read neighbouring words; a row of
+// it is read once for the workgroup's rows. The five vectors of a (token, head) lie side by side:
+// the scan stages them with straight copies.
 // ---------------------------------------------------------------------------------------
 #define DP_TOKENS 8
 #define DP_MAX_RANK 512
@@ -81,9 +84,8 @@ __device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-
 
 template <typename T>
 __global__ void __launch_bounds__(256)
-delta_prepare_kernel(const T* __restrict__ packed, long ld, int H, int D, int rank, WeightPtr w2, WeightPtr w0,
-                     WeightPtr a_bias, float decay_rate, float key_eps, const int* __restrict__ token_seq,
-                     float* __restrict__ coef, int n) {
+delta_prepare_kernel(const T* __restrict__ packed, long ld, int H, int D, int rank, WeightPtr w2t, WeightPtr w0,
+                     WeightPtr a_bias, float decay_rate, float key_eps, float* __restrict__ coef, int n) {
     __shared__ float th[DP_TOKENS][DP_MAX_RANK];
     __shared__ float inv_len[DP_TOKENS][DP_MAX_HEADS];
     const int inner = H * D;
@@ -118,139 +120,229 @@ delta_prepare_kernel(const T* __restrict__ packed, long ld, int H, int D, int ra
 #pragma unroll
     for (int tt = 0; tt < DP_TOKENS; ++tt) acc[tt] = 0.f;
     for (int j = 0; j < rank; ++j) {
-        const float w = w2.at((size_t)c * rank + j);
+        const float w = w2t.at((size_t)j * inner + c);
 #pragma unroll
         for (int tt = 0; tt < DP_TOKENS; ++tt) acc[tt] = fmaf(w, th[tt][j], acc[tt]);
     }
     const float b0 = w0.at(c), ab = a_bias.at(c);
-    const int hh = c / D - h_lo;
-    const size_t plane = (size_t)n * inner;
+    const int head = c / D, d = c % D;
+    const int hh = head - h_lo;
 #pragma unroll
     for (int tt = 0; tt < DP_TOKENS; ++tt) {
         if (tt >= nt) break;
         const size_t row = (size_t)(t0 + tt);
         const T* p = packed + row * ld;
-        const float u = to_f(p[inner + c]) * inv_len[tt][hh];
+        const float k = to_f(p[inner + c]);
+        const float u = k * inv_len[tt][hh];
         const float rate = sigmoid_f(to_f(p[4 * (size_t)inner + c]) + ab);
-        float* o = coef + row * inner + c;
+        float* o = coef + ((row * H + head) * 5) * (size_t)D + d;
         o[0] = expf(-decay_rate * sigmoid_f(acc[tt] + b0));
-        o[plane] = rate * u;
-        o[2 * plane] = u;
+        o[D] = rate * u;
+        o[2 * D] = u;
+        o[3 * D] = k;
+        o[4 * D] = to_f(p[c]);
     }
 }
 
-extern "C" int mv_delta_prepare(const void* packed, long ld, int n, int H, int D, int rank, const void* w2, const void* w0,
-                                const void* a_bias, int weight_dtype, float decay_rate, float key_eps,
-                                const int* token_seq, float* coef, int dtype, hipStream_t stream) {
+extern "C" int mv_delta_prepare(const void* packed, long ld, int n, int H, int D, int rank, const void* w2t, const void* w0,
+                                const void* a_bias, int weight_dtype, float decay_rate, float key_eps, float* coef,
+                                int dtype, hipStream_t stream) {
     MV_REQUIRE(n >= 0 && H > 0 && D > 0 && rank > 0, "delta_prepare: bad sizes n=%d H=%d D=%d rank=%d", n, H, D, rank);
     MV_REQUIRE(rank <= DP_MAX_RANK, "delta_prepare: rank %d exceeds the supported maximum %d", rank, DP_MAX_RANK);
     MV_REQUIRE(ld >= 5L * H * D + rank, "delta_prepare: rows of %ld columns do not hold 5 x %d + %d", ld, H * D, rank);
-    MV_REQUIRE(mv_valid_dtype(weight_dtype) && w2 && w0 && a_bias && coef, "delta_prepare: missing operand");
+    MV_REQUIRE(mv_valid_dtype(weight_dtype) && w2t && w0 && a_bias && coef, "delta_prepare: missing operand");
     MV_REQUIRE(key_eps > 0.f, "delta_prepare: key_eps must be positive");
     if (n == 0) return 0;
-    WeightPtr pw2{w2, weight_dtype}, pw0{w0, weight_dtype}, pab{a_bias, weight_dtype};
+    WeightPtr pw2{w2t, weight_dtype}, pw0{w0, weight_dtype}, pab{a_bias, weight_dtype};
     dim3 grid((n + DP_TOKENS - 1) / DP_TOKENS, (H * D + 255) / 256);
     MV_REQUIRE(grid.y <= 65535, "delta_prepare: too many channels");
     MV_DISPATCH_T(dtype, "delta_prepare",
                   hipLaunchKernelGGL(delta_prepare_kernel<T>, grid, dim3(256), 0, stream, (const T*)packed, ld, H, D,
-                                     rank, pw2, pw0, pab, decay_rate, key_eps, token_seq, coef, n));
+                                     rank, pw2, pw0, pab, decay_rate, key_eps, coef, n));
     return mv_check_launch("delta_prepare");
 }
 
 // ---------------------------------------------------------------------------------------
-// Delta rule, scan. A workgroup of 256 threads owns 64 value columns of one head of one request:
-// four neighbouring lanes share a column j, each keeps R rows of S[:, j] in registers (rows
-// sub*R .. sub*R+R-1, so D <= 4R; rows beyond D stay zero). Per token
-//     read = sum_i u_i S_ij            (R multiply-adds a lane, then a sum over the four lanes)
+// Delta rule, scan. A workgroup of 256 threads owns 256 / L value columns of one head of one
+// request: L neighbouring lanes share a column j, each keeps R rows of S[:, j] in registers (rows
+// sub*R .. sub*R+R-1, so D <= L*R; rows beyond D stay zero). Per token
+//     read = sum_i u_i S_ij            (R multiply-adds a lane, then a sum over the L lanes)
 //     S_ij = w_i S_ij - (a u)_i read + k_i v_j ;   o_j = sum_i r_i S_ij
-// The per-token vectors w, a*u, u, k, r (the same for every column) and v are staged in LDS,
-// 16 (or 8) tokens at a time. The request's state is read at the start and written at the end.
+// The per-token vectors w, a*u, u, k, r (the same for every column) and v are staged in LDS, a run of
+// tokens at a time, in two buffers: the next run's loads from memory are in flight while this run
+// is computed, and a token's vectors come from LDS into registers while the token before it is
+// computed. The request's state is read at the start and written at the end.
 // ---------------------------------------------------------------------------------------
-// lanes 4q .. 4q+3 end with the sum of their four values: two exchanges inside the quad (data-parallel
-// moves with the lane patterns [1,0,3,2] and [2,3,0,1]; nothing goes through LDS)
-__device__ __forceinline__ float quad_sum(float v) {
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+
+// the sum of a value over the L lanes that share a column (L = 4, 8 or 16 neighbouring lanes of a row
+// of 16): exchanges inside the row by data-parallel moves; every lane ends with the sum
+template <int L>
+__device__ __forceinline__ float lanes_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad [2,3,0,1]
+    if constexpr (L >= 8)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // mirror of 8
+    if constexpr (L >= 16)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // mirror of 16
     return v;
 }
 
-template <typename T, int R>
+template <int R>
+struct DeltaTokenRegs {
+    float w[R], au[R], u[R], k[R], r[R], v;
+};
+
+template <int R, int DPAD>
+__device__ __forceinline__ void delta_read_token(DeltaTokenRegs<R>& t, const float* vec, const float* vals, int sub, int col) {
+    // vec: [5][DPAD] of one token; vals: the token's value columns of this workgroup
+    const float* p = vec + sub * R;
+#pragma unroll
+    for (int e = 0; e < R; ++e) {
+        t.w[e] = p[e];
+        t.au[e] = p[DPAD + e];
+        t.u[e] = p[2 * DPAD + e];
+        t.k[e] = p[3 * DPAD + e];
+        t.r[e] = p[4 * DPAD + e];
+    }
+    t.v = vals[col];
+}
+
+template <int R, int L>
+__device__ __forceinline__ float delta_update(float (&s)[R], const DeltaTokenRegs<R>& t) {
+    float read = 0.f;
+#pragma unroll
+    for (int e = 0; e < R; ++e) read = fmaf(t.u[e], s[e], read);
+    read = lanes_sum<L>(read);
+    float o = 0.f;
+#pragma unroll
+    for (int e = 0; e < R; ++e) {
+        const float x = fmaf(t.w[e], s[e], fmaf(t.k[e], t.v, -t.au[e] * read));
+        s[e] = x;
+        o = fmaf(t.r[e], x, o);
+    }
+    return lanes_sum<L>(o);
+}
+
+// a lane's R rows of its column, between registers and the column's D floats in memory (rows
+// sub*R .. sub*R+R-1; rows beyond D are zero and are not stored)
+template <int R, bool STORE>
+__device__ __forceinline__ void delta_state_io(float (&s)[R], float* column, int sub, int D, bool live) {
+    const int i0 = sub * R;
+    if ((D & 3) == 0) {
+#pragma unroll
+        for (int e = 0; e < R; e += 4) {
+            float4* p = reinterpret_cast<float4*>(column + i0 + e);
+            const bool ok = live && i0 + e < D;
+            if constexpr (STORE) {
+                if (ok) *p = float4{s[e], s[e + 1], s[e + 2], s[e + 3]};
+            } else {
+                const float4 v = ok ? *p : float4{0.f, 0.f, 0.f, 0.f};
+                s[e] = v.x; s[e + 1] = v.y; s[e + 2] = v.z; s[e + 3] = v.w;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < R; ++e) {
+            const bool ok = live && i0 + e < D;
+            if constexpr (STORE) {
+                if (ok) column[i0 + e] = s[e];
+            } else {
+                s[e] = ok ? column[i0 + e] : 0.f;
+            }
+        }
+    }
+}
+
+template <typename T, int R, int L>
 __global__ void __launch_bounds__(256)
 delta_scan_kernel(const T* __restrict__ packed, long ld, const float* __restrict__ coef, float* __restrict__ state,
                   const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots, int H, int D,
                   float* __restrict__ out, int n) {
-    constexpr int DP = 4 * R;                       // padded key size
-    constexpr int DS_TOKENS = R > 32 ? 8 : 16;      // tokens staged at a time
-    __shared__ __attribute__((aligned(16))) float sv[5][DS_TOKENS][DP];   // w, a*u, u, k, r
-    __shared__ float svv[DS_TOKENS][64];
-    const int seq = blockIdx.x, head = blockIdx.y, j0 = blockIdx.z * 64;
+    constexpr int DPAD = L * R;                     // padded key size
+    constexpr int COLS = 256 / L;                   // value columns of a workgroup
+    constexpr int TT = DPAD > 128 ? 4 : (DPAD > 64 ? 8 : 16);          // tokens staged at a time
+    constexpr int NVEC = (TT * 5 * DPAD + 255) / 256;                   // staged words a thread brings in
+    constexpr int NVAL = (TT * COLS + 255) / 256;
+    __shared__ __attribute__((aligned(16))) float sv[2][TT][5][DPAD];
+    __shared__ float svv[2][TT][COLS];
+    const int seq = blockIdx.x, head = blockIdx.y, j0 = blockIdx.z * COLS;
     const int begin = cu_seqlens[seq], end = cu_seqlens[seq + 1];
     if (end <= begin) return;
     const int tid = threadIdx.x;
-    const int sub = tid & 3;
-    const int col = tid >> 2;                        // 0..63
+    const int sub = tid % L;
+    const int col = tid / L;
     const int j = j0 + col;
     const bool live = j < D;
     const int inner = H * D;
-    const size_t plane = (size_t)n * inner;
-    float* S = state + ((size_t)state_slots[seq] * H + head) * (size_t)D * D;
+    // the state of a head is stored column by column, S[j][i]: a lane's rows are neighbours in memory
+    float* S = state + ((size_t)state_slots[seq] * H + head) * (size_t)D * D + (size_t)(live ? j : 0) * D;
     float s[R];
+    delta_state_io<R, false>(s, S, sub, D, live);
+    // a run of tokens from memory into registers, and from there into an LDS buffer
+    float gv[NVEC], gx[NVAL];
+    auto fetch = [&](int base) {
+        const int nt = min(TT, end - base);
 #pragma unroll
-    for (int e = 0; e < R; ++e) {
-        const int i = sub * R + e;
-        s[e] = (live && i < D) ? S[(size_t)i * D + j] : 0.f;
-    }
-    for (int base = begin; base < end; base += DS_TOKENS) {
-        const int nt = min(DS_TOKENS, end - base);
-        __syncthreads();
-        for (int x = tid; x < nt * DP; x += 256) {
-            const int tt = x / DP, i = x % DP;
-            const size_t row = (size_t)(base + tt);
-            float w = 0.f, au = 0.f, u = 0.f, k = 0.f, r = 0.f;
-            if (i < D) {
-                const size_t c = row * inner + (size_t)head * D + i;
-                w = coef[c];
-                au = coef[plane + c];
-                u = coef[2 * plane + c];
-                const T* p = packed + row * ld + (size_t)head * D + i;
-                r = to_f(p[0]);
-                k = to_f(p[inner]);
+        for (int q = 0; q < NVEC; ++q) {
+            const int x = tid + q * 256;
+            const int tt = x / (5 * DPAD), rem = x % (5 * DPAD), a = rem / DPAD, i = rem % DPAD;
+            gv[q] = (tt < nt && i < D) ? coef[(((size_t)(base + tt) * H + head) * 5 + a) * D + i] : 0.f;
+        }
+#pragma unroll
+        for (int q = 0; q < NVAL; ++q) {
+            const int x = tid + q * 256;
+            const int tt = x / COLS, jj = x % COLS;
+            gx[q] = (tt < nt && tt < TT && j0 + jj < D)
+                        ? to_f(packed[(size_t)(base + tt) * ld + 2 * (size_t)inner + (size_t)head * D + j0 + jj]) : 0.f;
+        }
+    };
+    auto stash = [&](int buf) {
+        float* dst = &sv[buf][0][0][0];
+#pragma unroll
+        for (int q = 0; q < NVEC; ++q) {
+            const int x = tid + q * 256;
+            if (x < TT * 5 * DPAD) dst[x] = gv[q];
+        }
+        float* dv = &svv[buf][0][0];
+#pragma unroll
+        for (int q = 0; q < NVAL; ++q) {
+            const int x = tid + q * 256;
+            if (x < TT * COLS) dv[x] = gx[q];
+        }
+    };
+    fetch(begin);
+    stash(0);
+    __syncthreads();
+    int buf = 0;
+    for (int base = begin; base < end; base += TT, buf ^= 1) {
+        const int nt = min(TT, end - base);
+        const bool more = base + TT < end;
+        if (more) fetch(base + TT);                  // in flight while this run is computed
+        DeltaTokenRegs<R> ta, tb;
+        delta_read_token<R, DPAD>(ta, &sv[buf][0][0][0], &svv[buf][0][0], sub, col);
+        for (int tt = 0; tt < nt; tt += 2) {
+            if (tt + 1 < nt) delta_read_token<R, DPAD>(tb, &sv[buf][tt + 1][0][0], &svv[buf][tt + 1][0], sub, col);
+            const float o0 = delta_update<R, L>(s, ta);
+            if (live && sub == 0) out[(size_t)(base + tt) * inner + (size_t)head * D + j] = o0;
+            if (tt + 1 < nt) {
+                if (tt + 2 < nt) delta_read_token<R, DPAD>(ta, &sv[buf][tt + 2][0][0], &svv[buf][tt + 2][0], sub, col);
+                const float o1 = delta_update<R, L>(s, tb);
+                if (live && sub == 0) out[(size_t)(base + tt + 1) * inner + (size_t)head * D + j] = o1;
             }
-            sv[0][tt][i] = w; sv[1][tt][i] = au; sv[2][tt][i] = u; sv[3][tt][i] = k; sv[4][tt][i] = r;
         }
-        for (int x = tid; x < nt * 64; x += 256) {
-            const int tt = x / 64, jj = x % 64;
-            svv[tt][jj] = (j0 + jj < D) ? to_f(packed[(size_t)(base + tt) * ld + 2 * (size_t)inner + (size_t)head * D + j0 + jj])
-                                        : 0.f;
-        }
+        if (more) stash(buf ^ 1);                    // nobody reads that buffer: its run was computed before the last barrier
         __syncthreads();
-        for (int tt = 0; tt < nt; ++tt) {
-            const float* w = &sv[0][tt][sub * R];
-            const float* au = &sv[1][tt][sub * R];
-            const float* u = &sv[2][tt][sub * R];
-            const float* k = &sv[3][tt][sub * R];
-            const float* r = &sv[4][tt][sub * R];
-            float read = 0.f;
-#pragma unroll
-            for (int e = 0; e < R; ++e) read = fmaf(u[e], s[e], read);
-            read = quad_sum(read);
-            const float vj = svv[tt][col];
-            float o = 0.f;
-#pragma unroll
-            for (int e = 0; e < R; ++e) {
-                const float x = fmaf(w[e], s[e], fmaf(k[e], vj, -au[e] * read));
-                s[e] = x;
-                o = fmaf(r[e], x, o);
-            }
-            o = quad_sum(o);
-            if (live && sub == 0) out[(size_t)(base + tt) * inner + (size_t)head * D + j] = o;
-        }
     }
-#pragma unroll
-    for (int e = 0; e < R; ++e) {
-        const int i = sub * R + e;
-        if (live && i < D) S[(size_t)i * D + j] = s[e];
-    }
+    delta_state_io<R, true>(s, S, sub, D, live);
+}
+
+// how a head of size D is dealt out: (rows a lane keeps, lanes a column); 0 when D is not served
+static void delta_scan_shape(int D, int& R, int& L) {
+    if (D <= 16) { R = 4; L = 4; }
+    else if (D <= 32) { R = 8; L = 4; }
+    else if (D <= 64) { R = 8; L = 8; }
+    else if (D <= 128) { R = 8; L = 16; }
+    else { R = 16; L = 16; }
 }
 
 extern "C" int mv_delta_scan(const void* packed, long ld, const float* coef, float* state, const int* cu_seqlens,
@@ -260,26 +352,153 @@ extern "C" int mv_delta_scan(const void* packed, long ld, const float* coef, flo
     MV_REQUIRE(D <= 256, "delta_scan: head size %d exceeds the supported maximum 256", D);
     MV_REQUIRE(ld >= 3L * H * D, "delta_scan: rows of %ld columns do not hold r, k and v of %d", ld, H * D);
     MV_REQUIRE(packed && coef && state && cu_seqlens && state_slots && out, "delta_scan: missing operand");
-    MV_REQUIRE(H <= 65535 && (D + 63) / 64 <= 65535, "delta_scan: too many heads");
+    int R = 0, L = 0;
+    delta_scan_shape(D, R, L);
+    const int cols = 256 / L;
+    MV_REQUIRE(H <= 65535 && (D + cols - 1) / cols <= 65535, "delta_scan: too many heads");
     if (n == 0 || n_seqs == 0) return 0;
-    dim3 grid(n_seqs, H, (D + 63) / 64);
-#define DS_LAUNCH(R)                                                                                                 \
-    MV_DISPATCH_T(dtype, "delta_scan",                                                                               \
-                  hipLaunchKernelGGL((delta_scan_kernel<T, R>), grid, dim3(256), 0, stream, (const T*)packed, ld, coef, \
+    dim3 grid(n_seqs, H, (D + cols - 1) / cols);
+#define DS_LAUNCH(RR, LL)                                                                                                \
+    MV_DISPATCH_T(dtype, "delta_scan",                                                                                   \
+                  hipLaunchKernelGGL((delta_scan_kernel<T, RR, LL>), grid, dim3(256), 0, stream, (const T*)packed, ld, coef, \
                                      state, cu_seqlens, state_slots, H, D, out, n))
-    if (D <= 16) {
-        DS_LAUNCH(4);
-    } else if (D <= 32) {
-        DS_LAUNCH(8);
-    } else if (D <= 64) {
-        DS_LAUNCH(16);
-    } else if (D <= 128) {
-        DS_LAUNCH(32);
+    if (R == 4 && L == 4) {
+        DS_LAUNCH(4, 4);
+    } else if (R == 8 && L == 4) {
+        DS_LAUNCH(8, 4);
+    } else if (R == 8 && L == 8) {
+        DS_LAUNCH(8, 8);
+    } else if (R == 8 && L == 16) {
+        DS_LAUNCH(8, 16);
     } else {
-        DS_LAUNCH(64);
+        DS_LAUNCH(16, 16);
     }
 #undef DS_LAUNCH
     return mv_check_launch("delta_scan");
+}
+
+// ---------------------------------------------------------------------------------------
+// Delta rule, a step of single tokens: prepare, the recurrence and finish for one (row, head) in one
+// workgroup. Row t is the one new token of request token_seq[t] (a padding row, < 0, gives zeros and
+// touches no state). The head's columns are taken 256 / L at a time with the lanes laid out as in the
+// scan; the additions are the scan's and the other kernels', in the same order, so a token computed here
+// has the bits it would have as a prompt's last token.
+// ---------------------------------------------------------------------------------------
+template <typename T, int R, int L>
+__global__ void __launch_bounds__(256)
+delta_step_kernel(const T* __restrict__ packed, long ld, int H, int D, int rank, WeightPtr w2t, WeightPtr w0,
+                  WeightPtr a_bias, float decay_rate, float key_eps, float* __restrict__ state,
+                  const int* __restrict__ token_seq, const int* __restrict__ state_slots, WeightPtr norm_w, float eps,
+                  T* __restrict__ out, long ldo) {
+    constexpr int DPAD = L * R;
+    constexpr int COLS = 256 / L;
+    __shared__ float th[DP_MAX_RANK];
+    __shared__ __attribute__((aligned(16))) float vec[5][DPAD];
+    __shared__ float vals[DPAD];
+    __shared__ float outs[DPAD];
+    __shared__ float red[8];
+    const int t = blockIdx.x, head = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int lane = tid % MV_WAVE, wave = tid / MV_WAVE;
+    const int inner = H * D;
+    const int seq = token_seq[t];
+    T* y = out + (size_t)t * ldo + (size_t)head * D;
+    if (seq < 0) {
+        for (int d = tid; d < D; d += 256) y[d] = from_f<T>(0.f);
+        return;
+    }
+    const T* p = packed + (size_t)t * ld;
+    for (int j = tid; j < rank; j += 256) th[j] = tanhf(to_f(p[5 * (size_t)inner + j]));
+    // the head's key and its length (the sum runs as the prepare kernel's: a wave over the head, lane by lane)
+    if (wave == 0) {
+        float ss = 0.f;
+        for (int d = lane; d < D; d += MV_WAVE) {
+            const float v = to_f(p[inner + head * D + d]);
+            ss = fmaf(v, v, ss);
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) red[0] = 1.f / sqrtf(ss + key_eps);
+    }
+    __syncthreads();
+    for (int d = tid; d < DPAD; d += 256) {
+        float w = 0.f, au = 0.f, u = 0.f, k = 0.f, r = 0.f, v = 0.f;
+        if (d < D) {
+            const int cc = head * D + d;
+            float acc = 0.f;
+            for (int j = 0; j < rank; ++j) acc = fmaf(w2t.at((size_t)j * inner + cc), th[j], acc);
+            k = to_f(p[inner + cc]);
+            u = k * red[0];
+            au = sigmoid_f(to_f(p[4 * (size_t)inner + cc]) + a_bias.at(cc)) * u;
+            w = expf(-decay_rate * sigmoid_f(acc + w0.at(cc)));
+            r = to_f(p[cc]);
+            v = to_f(p[2 * (size_t)inner + cc]);
+        }
+        vec[0][d] = w; vec[1][d] = au; vec[2][d] = u; vec[3][d] = k; vec[4][d] = r;
+        vals[d] = v;
+    }
+    __syncthreads();
+    const int sub = tid % L, col = tid / L;
+    float* S0 = state + ((size_t)state_slots[seq] * H + head) * (size_t)D * D;
+    for (int j0 = 0; j0 < D; j0 += COLS) {
+        const int j = j0 + col;
+        const bool live = j < D;
+        float* S = S0 + (size_t)(live ? j : 0) * D;
+        float s[R];
+        delta_state_io<R, false>(s, S, sub, D, live);
+        DeltaTokenRegs<R> tk;
+        delta_read_token<R, DPAD>(tk, &vec[0][0], vals, sub, live ? j : 0);
+        const float o = delta_update<R, L>(s, tk);
+        delta_state_io<R, true>(s, S, sub, D, live);
+        if (live && sub == 0) outs[j] = o;
+    }
+    __syncthreads();
+    // the head's root mean square (a wave over the head, lane by lane, as the finish kernel sums), weight, gate
+    if (wave == 0) {
+        float ss = 0.f;
+        for (int d = lane; d < D; d += MV_WAVE) ss = fmaf(outs[d], outs[d], ss);
+        ss = wave_sum(ss);
+        if (lane == 0) red[1] = 1.f / sqrtf(ss / (float)D + eps);
+    }
+    __syncthreads();
+    for (int d = tid; d < D; d += 256) {
+        const int cc = head * D + d;
+        y[d] = from_f<T>(outs[d] * red[1] * norm_w.at(cc) * sigmoid_f(to_f(p[3 * (size_t)inner + cc])));
+    }
+}
+
+extern "C" int mv_delta_step(const void* packed, long ld, int n, int H, int D, int rank, const void* w2t, const void* w0,
+                             const void* a_bias, const void* norm_w, int weight_dtype, float decay_rate, float key_eps,
+                             float eps, float* state, const int* token_seq, const int* state_slots, void* out, long ldo,
+                             int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && H > 0 && D > 0 && rank > 0, "delta_step: bad sizes n=%d H=%d D=%d rank=%d", n, H, D, rank);
+    MV_REQUIRE(rank <= DP_MAX_RANK && D <= 256, "delta_step: rank %d or head size %d exceed what is served", rank, D);
+    MV_REQUIRE(ld >= 5L * H * D + rank && ldo >= (long)H * D, "delta_step: row pitches too small");
+    MV_REQUIRE(mv_valid_dtype(weight_dtype) && packed && w2t && w0 && a_bias && norm_w && state && token_seq && state_slots && out,
+               "delta_step: missing operand");
+    MV_REQUIRE(key_eps > 0.f && eps > 0.f && H <= 65535, "delta_step: bad constants");
+    if (n == 0) return 0;
+    int R = 0, L = 0;
+    delta_scan_shape(D, R, L);
+    WeightPtr pw2{w2t, weight_dtype}, pw0{w0, weight_dtype}, pab{a_bias, weight_dtype}, pn{norm_w, weight_dtype};
+    dim3 grid(n, H);
+#define DT_LAUNCH(RR, LL)                                                                                                   \
+    MV_DISPATCH_T(dtype, "delta_step",                                                                                      \
+                  hipLaunchKernelGGL((delta_step_kernel<T, RR, LL>), grid, dim3(256), 0, stream, (const T*)packed, ld, H, D,  \
+                                     rank, pw2, pw0, pab, decay_rate, key_eps, state, token_seq, state_slots, pn, eps,      \
+                                     (T*)out, ldo))
+    if (R == 4 && L == 4) {
+        DT_LAUNCH(4, 4);
+    } else if (R == 8 && L == 4) {
+        DT_LAUNCH(8, 4);
+    } else if (R == 8 && L == 8) {
+        DT_LAUNCH(8, 8);
+    } else if (R == 8 && L == 16) {
+        DT_LAUNCH(8, 16);
+    } else {
+        DT_LAUNCH(16, 16);
+    }
+#undef DT_LAUNCH
+    return mv_check_launch("delta_step");
 }
 
 // ---------------------------------------------------------------------------------------

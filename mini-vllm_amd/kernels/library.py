@@ -48,9 +48,13 @@ _SIGNATURES = {
     # h, ldh, out, ldo, mix, mix_dtype, state, token_seq, cu_seqlens, state_slots, n, width, dtype, stream
     "mv_token_shift": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_int, c_int, c_int, c_void_p]),
-    # packed, ld, n, H, D, rank, w2, w0, a_bias, weight_dtype, decay_rate, key_eps, token_seq, coef, dtype, stream
+    # packed, ld, n, H, D, rank, w2t, w0, a_bias, weight_dtype, decay_rate, key_eps, coef, dtype, stream
     "mv_delta_prepare": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
-                                 c_float, c_float, c_void_p, c_void_p, c_int, c_void_p]),
+                                 c_float, c_float, c_void_p, c_int, c_void_p]),
+    # packed, ld, n, H, D, rank, w2t, w0, a_bias, norm_w, weight_dtype, decay_rate, key_eps, eps, state, token_seq,
+    # state_slots, out, ldo, dtype, stream
+    "mv_delta_step": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                              c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_int, c_void_p]),
     # packed, ld, coef, state, cu_seqlens, state_slots, n_seqs, n, H, D, out, dtype, stream
     "mv_delta_scan": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                               c_void_p, c_int, c_void_p]),

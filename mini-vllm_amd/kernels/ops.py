@@ -467,52 +467,82 @@ class Ops:
                       out.stride(0) if n > 1 else w, mix.data_ptr(), _weight_code(mix, "shift weight"), state.data_ptr(),
                       token_seq.data_ptr(), cu_seqlens.data_ptr(), state_slots.data_ptr(), n, w, self.code, self._stream())
 
-    def delta_prepare(self, packed: torch.Tensor, heads: int, dim: int, rank: int, w2: torch.Tensor, w0: torch.Tensor,
-                      a_bias: torch.Tensor, decay_rate: float, key_eps: float, token_seq: torch.Tensor,
-                      coef: torch.Tensor) -> None:
+    def _delta_weights(self, heads: int, dim: int, rank: int, w2t: torch.Tensor, w0: torch.Tensor, a_bias: torch.Tensor,
+                       what: str) -> int:
+        inner = heads * dim
+        for t, shape, name in ((w2t, (rank, inner), "w2 (transposed)"), (w0, (inner,), "w0"), (a_bias, (inner,), "a_bias")):
+            _dev(t, name)
+            if tuple(t.shape) != shape or not t.is_contiguous() or t.dtype != w2t.dtype:
+                raise KernelLibraryError(f"{what}: {name} must be a contiguous {shape} tensor of w2's dtype")
+        return _weight_code(w2t, "w2")
+
+    def delta_prepare(self, packed: torch.Tensor, heads: int, dim: int, rank: int, w2t: torch.Tensor, w0: torch.Tensor,
+                      a_bias: torch.Tensor, decay_rate: float, key_eps: float, coef: torch.Tensor) -> None:
         """From rows [r | k | v | g | a | w1] (heads*dim columns each, ``rank`` for w1) the float32
-        coefficients of the delta rule, coef [3, n, heads*dim]: the decay
+        vectors of the delta rule, coef [n, heads, 5, dim]: the decay
         exp(-decay_rate * sigmoid(w2 tanh(w1) + w0)), rate * unit key with rate = sigmoid(a + a_bias),
-        and the unit key k / sqrt(sum(k^2) + key_eps) of each head."""
+        the unit key k / sqrt(sum(k^2) + key_eps) of each head, k and r. ``w2t`` is w2 transposed, [rank, heads*dim]."""
         self._act(packed, "delta rows")
         n, inner = packed.shape[0], heads * dim
         if packed.dim() != 2 or packed.stride(1) != 1 or packed.shape[1] < 5 * inner + rank:
             raise KernelLibraryError(f"delta_prepare: rows {tuple(packed.shape)} do not hold 5 x {inner} + {rank} columns")
-        if coef.dtype != torch.float32 or tuple(coef.shape) != (3, n, inner) or not coef.is_contiguous():
-            raise KernelLibraryError(f"delta_prepare: coefficients must be float32 [3, {n}, {inner}]")
-        for t, shape, what in ((w2, (inner, rank), "w2"), (w0, (inner,), "w0"), (a_bias, (inner,), "a_bias")):
-            _dev(t, what)
-            if tuple(t.shape) != shape or not t.is_contiguous() or t.dtype != w2.dtype:
-                raise KernelLibraryError(f"delta_prepare: {what} must be a contiguous {shape} tensor of w2's dtype")
-        self._ints(n, token_seq=(token_seq, n))
-        self._note("mv_delta_prepare", n * (2 * inner + rank) * packed.element_size() + self._size(w2, coef), 2 * n * inner * rank)
+        if coef.dtype != torch.float32 or tuple(coef.shape) != (n, heads, 5, dim) or not coef.is_contiguous():
+            raise KernelLibraryError(f"delta_prepare: coefficients must be float32 [{n}, {heads}, 5, {dim}]")
+        wcode = self._delta_weights(heads, dim, rank, w2t, w0, a_bias, "delta_prepare")
+        self._note("mv_delta_prepare", n * (3 * inner + rank) * packed.element_size() + self._size(w2t, coef), 2 * n * inner * rank)
         self.lib.call("mv_delta_prepare", packed.data_ptr(), packed.stride(0) if n > 1 else packed.shape[1], n, heads, dim,
-                      rank, w2.data_ptr(), w0.data_ptr(), a_bias.data_ptr(), _weight_code(w2, "w2"), float(decay_rate),
-                      float(key_eps), token_seq.data_ptr(), coef.data_ptr(), self.code, self._stream())
+                      rank, w2t.data_ptr(), w0.data_ptr(), a_bias.data_ptr(), wcode, float(decay_rate),
+                      float(key_eps), coef.data_ptr(), self.code, self._stream())
+
+    def _delta_state(self, state: torch.Tensor, heads: int, dim: int, what: str) -> None:
+        _dev(state, "delta state")
+        if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, dim) or not state.is_contiguous():
+            raise KernelLibraryError(f"{what}: the state must be float32 [slots, {heads}, {dim}, {dim}]")
 
     def delta_scan(self, packed: torch.Tensor, coef: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor,
                    state_slots: torch.Tensor, n_seqs: int, heads: int, dim: int, out: torch.Tensor) -> None:
         """The delta rule over the step's rows, request by request (rows cu_seqlens[s] .. cu_seqlens[s+1]
         of request s, state row state_slots[s]): S <- diag(w) S - (a*u)(u^T S) + k v^T, out = S^T r, with
-        r, k, v from the packed rows and w, a*u, u from ``coef``. state float32 [slots, heads, dim, dim] is
-        read and left advanced; out float32 [n, heads*dim]."""
+        v from the packed rows and w, a*u, u, k, r from ``coef``. state float32 [slots, heads, dim, dim]
+        holds each head's matrix column by column (state[.., j, i] = S[i][j], i the key channel); it is
+        read and left advanced. out float32 [n, heads*dim]."""
         self._act(packed, "delta rows")
         n, inner = packed.shape[0], heads * dim
-        if coef.dtype != torch.float32 or tuple(coef.shape) != (3, n, inner) or not coef.is_contiguous():
-            raise KernelLibraryError(f"delta_scan: coefficients must be float32 [3, {n}, {inner}]")
+        if coef.dtype != torch.float32 or tuple(coef.shape) != (n, heads, 5, dim) or not coef.is_contiguous():
+            raise KernelLibraryError(f"delta_scan: coefficients must be float32 [{n}, {heads}, 5, {dim}]")
         if out.dtype != torch.float32 or tuple(out.shape) != (n, inner) or not out.is_contiguous():
             raise KernelLibraryError(f"delta_scan: the output must be float32 [{n}, {inner}]")
-        _dev(state, "delta state")
-        if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, dim) or not state.is_contiguous():
-            raise KernelLibraryError(f"delta_scan: the state must be float32 [slots, {heads}, {dim}, {dim}]")
+        self._delta_state(state, heads, dim, "delta_scan")
         if packed.dim() != 2 or packed.stride(1) != 1 or packed.shape[1] < 3 * inner:
             raise KernelLibraryError(f"delta_scan: rows {tuple(packed.shape)} do not hold r, k and v")
         self._ints(n, cu_seqlens=(cu_seqlens, n_seqs + 1), state_slots=(state_slots, n_seqs))
-        self._note("mv_delta_scan", 3 * n * inner * packed.element_size() + self._size(coef, out)
+        self._note("mv_delta_scan", n * inner * packed.element_size() + self._size(coef, out)
                    + 2 * min(n_seqs, max(n, 1)) * inner * dim * 4, 8 * n * inner * dim)
         self.lib.call("mv_delta_scan", packed.data_ptr(), packed.stride(0) if n > 1 else packed.shape[1], coef.data_ptr(),
                       state.data_ptr(), cu_seqlens.data_ptr(), state_slots.data_ptr(), n_seqs, n, heads, dim,
                       out.data_ptr(), self.code, self._stream())
+
+    def delta_step(self, packed: torch.Tensor, heads: int, dim: int, rank: int, w2t: torch.Tensor, w0: torch.Tensor,
+                   a_bias: torch.Tensor, norm_weight: torch.Tensor, decay_rate: float, key_eps: float, eps: float,
+                   state: torch.Tensor, token_seq: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor) -> None:
+        """``delta_prepare``, ``delta_scan`` and ``delta_finish`` in one kernel for a step in which every
+        request brings one token: row t belongs to request token_seq[t] (negative: a padding row)."""
+        self._act(packed, "delta rows"); self._act(out, "delta output"); _dev(norm_weight, "delta norm weight")
+        n, inner = packed.shape[0], heads * dim
+        if packed.dim() != 2 or packed.stride(1) != 1 or packed.shape[1] < 5 * inner + rank:
+            raise KernelLibraryError(f"delta_step: rows {tuple(packed.shape)} do not hold 5 x {inner} + {rank} columns")
+        if tuple(out.shape) != (n, inner) or out.stride(1) != 1 or norm_weight.numel() != inner \
+                or not norm_weight.is_contiguous() or norm_weight.dtype != w2t.dtype:
+            raise KernelLibraryError("delta_step: output or norm weight do not fit")
+        wcode = self._delta_weights(heads, dim, rank, w2t, w0, a_bias, "delta_step")
+        self._delta_state(state, heads, dim, "delta_step")
+        self._ints(n, token_seq=(token_seq, n), state_slots=(state_slots, 1))
+        self._note("mv_delta_step", n * (5 * inner + rank) * packed.element_size() + self._size(w2t, out)
+                   + 2 * n * inner * dim * 4, 8 * n * inner * dim + 2 * n * inner * rank)
+        self.lib.call("mv_delta_step", packed.data_ptr(), packed.stride(0) if n > 1 else packed.shape[1], n, heads, dim, rank,
+                      w2t.data_ptr(), w0.data_ptr(), a_bias.data_ptr(), norm_weight.data_ptr(), wcode, float(decay_rate),
+                      float(key_eps), float(eps), state.data_ptr(), token_seq.data_ptr(), state_slots.data_ptr(),
+                      out.data_ptr(), out.stride(0) if n > 1 else inner, self.code, self._stream())
 
     def delta_finish(self, raw: torch.Tensor, packed: torch.Tensor, weight: torch.Tensor, heads: int, dim: int,
                      eps: float, out: torch.Tensor) -> None:

@@ -10,12 +10,13 @@ rate a per key channel, and the unit key u = k / sqrt(sum(k^2) + key_eps):
 
 Each head's o is divided by its root mean square, the heads are concatenated, multiplied by a
 weight over all heads' channels and by sigmoid(Wg h), and projected back to the model's width.
-S starts at zero and is float32 [heads, head_dim, head_dim] per request (``state``), whatever the
-activation type; decays, rates, unit keys and the recurrence itself are float32 too.
+S starts at zero and is float32 [heads, head_dim, head_dim] per request (``state``, each head's matrix
+stored column by column), whatever the activation type; decays, rates, unit keys and the recurrence
+itself are float32 too.
 
 r, k, v, g, a and W1 read the same input and are one packed product; everything between that
 product and the output projection is three kernels (prepare, scan, finish) for any mix of prompt
-portions and single tokens.
+portions and single tokens, and one kernel for a step in which every request brings one token.
 """
 from __future__ import annotations
 
@@ -80,7 +81,9 @@ class DeltaRule(Mixer):
             blocks.append(torch.zeros((pad, spec.hidden_size), dtype=blocks[0].dtype, device=blocks[0].device))
         self.w_packed = torch.cat(blocks, dim=0).contiguous()
         self.width = self.w_packed.shape[0]
-        self.w2, self.w0, self.a_bias = tensors["w2"], tensors["w0"], tensors["a_bias"]
+        # transposed, [rank, heads * head_dim]: neighbouring channels then read neighbouring words
+        self.w2_t = tensors["w2"].t().contiguous()
+        self.w0, self.a_bias = tensors["w0"], tensors["a_bias"]
         self.norm, self.w_o = tensors["norm"], tensors["o"]
 
     def forward(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
@@ -88,14 +91,21 @@ class DeltaRule(Mixer):
         n, inner = x.shape[0], spec.inner
         packed = ws.get("delta.packed", (n, self.width), rt.dtype)
         ops.gemm(x, self.w_packed, packed)
-        # float32 [3, n, inner]: decay, rate * unit key, unit key
-        coef = ws.get("delta.coef", (3, n, inner), torch.float32)
-        ops.delta_prepare(packed, spec.num_heads, spec.head_dim, spec.decay_rank, self.w2, self.w0, self.a_bias,
-                          spec.decay_rate, spec.key_eps, ctx.token_seq, coef)
-        raw = ws.get("delta.raw", (n, inner), torch.float32)
-        ops.delta_scan(packed, coef, ctx.state(call), ctx.cu_seqlens, ctx.state_slots, ctx.n_seqs,
-                       spec.num_heads, spec.head_dim, raw)
         gated = ws.get("delta.gated", (n, inner), rt.dtype)
-        ops.delta_finish(raw, packed, self.norm, spec.num_heads, spec.head_dim, spec.out_norm_eps, gated)
+        plan = ctx.attention_plan
+        if plan is not None and plan.decode_only:
+            # every request brings one token: the three kernels below as one
+            ops.delta_step(packed, spec.num_heads, spec.head_dim, spec.decay_rank, self.w2_t, self.w0, self.a_bias,
+                           self.norm, spec.decay_rate, spec.key_eps, spec.out_norm_eps, ctx.state(call), ctx.token_seq,
+                           ctx.state_slots, gated)
+        else:
+            # float32 [n, heads, 5, head_dim]: decay, rate * unit key, unit key, key, receptance
+            coef = ws.get("delta.coef", (n, spec.num_heads, 5, spec.head_dim), torch.float32)
+            ops.delta_prepare(packed, spec.num_heads, spec.head_dim, spec.decay_rank, self.w2_t, self.w0, self.a_bias,
+                              spec.decay_rate, spec.key_eps, coef)
+            raw = ws.get("delta.raw", (n, inner), torch.float32)
+            ops.delta_scan(packed, coef, ctx.state(call), ctx.cu_seqlens, ctx.state_slots, ctx.n_seqs,
+                           spec.num_heads, spec.head_dim, raw)
+            ops.delta_finish(raw, packed, self.norm, spec.num_heads, spec.head_dim, spec.out_norm_eps, gated)
         y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
         return ops.gemm(gated, self.w_o, y, defer_sum=True) or y

@@ -94,15 +94,23 @@ def delta_plain(packed, t, H, D, rank, eps, states):
     return raw.reshape(n, inner), gated, torch.stack(final)
 
 
-def run_delta(ops, packed, t, H, D, rank, eps, state, q_lens, slots, pad_rows=0, pad_seqs=0):
+def run_delta(ops, packed, t, H, D, rank, eps, state, q_lens, slots, pad_rows=0, pad_seqs=0, fused=False):
+    """``state`` [slots, H, D, D] holds each head's matrix column by column (the transpose of the plain S).
+    ``fused``: the one kernel for steps of single tokens (every q_len must be 1); it returns no raw rows."""
     n, inner = packed.shape[0], H * D
     tsq, cu, sl = step_ints(q_lens, slots, pad_rows, pad_seqs)
     dev = {k: v.to(DEV) for k, v in t.items()}
-    coef = torch.empty(3, n, inner, dtype=torch.float32, device=DEV)
-    raw = torch.zeros(n, inner, dtype=torch.float32, device=DEV)
+    w2t = dev["w2"].t().contiguous()
     out = torch.empty(n, inner, dtype=packed.dtype, device=DEV)
     p = packed.to(DEV)
-    ops.delta_prepare(p, H, D, rank, dev["w2"], dev["w0"], dev["a_bias"], plain.DECAY_RATE, plain.DELTA_KEY_EPS, tsq, coef)
+    if fused:
+        ops.delta_step(p, H, D, rank, w2t, dev["w0"], dev["a_bias"], dev["norm"], plain.DECAY_RATE, plain.DELTA_KEY_EPS,
+                       eps, state, tsq, sl, out)
+        torch.cuda.synchronize()
+        return None, out
+    coef = torch.empty(n, H, 5, D, dtype=torch.float32, device=DEV)
+    raw = torch.zeros(n, inner, dtype=torch.float32, device=DEV)
+    ops.delta_prepare(p, H, D, rank, w2t, dev["w0"], dev["a_bias"], plain.DECAY_RATE, plain.DELTA_KEY_EPS, coef)
     ops.delta_scan(p, coef, state, cu, sl, len(q_lens) + pad_seqs, H, D, raw)
     ops.delta_finish(raw, p, dev["norm"], H, D, eps, out)
     torch.cuda.synchronize()
@@ -121,17 +129,43 @@ def test_delta_rule_mixed_step(dtype, H, D, rank):
     packed, t = delta_inputs(n + 3, H, D, rank, seed=H * 1000 + D, dtype=dtype)
     g = torch.Generator().manual_seed(5)
     state = torch.randn(6, H, D, D, generator=g) * 0.3
-    dstate = state.to(DEV).clone()
+    dstate = state.transpose(-1, -2).contiguous().to(DEV)
     raw, out = run_delta(ops, packed, t, H, D, rank, eps, dstate, q_lens, slots, pad_rows=3, pad_seqs=2)
     base = 0
     for q, slot in zip(q_lens, slots):
         want_raw, want, final = delta_plain(packed[base:base + q], t, H, D, rank, eps, state[slot])
         close(raw[base:base + q], want_raw, 2e-5, f"scan of request in slot {slot}")
         close(out[base:base + q], want, 2e-5 if dtype == torch.float32 else 8e-3, "finished rows")
-        close(dstate[slot], final, 2e-5, "state after the step")
+        close(dstate[slot].transpose(-1, -2), final, 2e-5, "state after the step")
         base += q
     for slot in (2, 5):
-        assert torch.equal(dstate[slot].cpu(), state[slot])
+        assert torch.equal(dstate[slot].transpose(-1, -2).cpu(), state[slot])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H, D, rank", [(2, 16, 6), (3, 24, 5), (1, 40, 3), (4, 64, 32), (2, 128, 16), (1, 200, 4),
+                                        (5, 8, 1)])
+def test_delta_rule_step_of_single_tokens(dtype, H, D, rank):
+    """Five requests with one token each (slots out of order, a padding row between them): the one fused
+    kernel against the plain recurrence, and against the three kernels it stands for."""
+    ops = ops_for(dtype)
+    slots, eps = [3, 0, 4, 1, 5], 1e-5
+    packed, t = delta_inputs(7, H, D, rank, seed=H * 77 + D, dtype=dtype)
+    g = torch.Generator().manual_seed(6)
+    state = torch.randn(7, H, D, D, generator=g) * 0.3
+    fused_state = state.transpose(-1, -2).contiguous().to(DEV)
+    three_state = fused_state.clone()
+    _, fused = run_delta(ops, packed, t, H, D, rank, eps, fused_state, [1] * 5, slots, pad_rows=2, fused=True)
+    _, three = run_delta(ops, packed, t, H, D, rank, eps, three_state, [1] * 5, slots, pad_rows=2)
+    for row, slot in enumerate(slots):
+        _, want, final = delta_plain(packed[row:row + 1], t, H, D, rank, eps, state[slot])
+        close(fused[row:row + 1], want, 2e-5 if dtype == torch.float32 else 8e-3, f"row {row}")
+        close(fused_state[slot].transpose(-1, -2), final, 2e-5, "state after the step")
+    close(fused[:5], three[:5].double(), 1e-6 if dtype == torch.float32 else 8e-3, "fused against three kernels")
+    close(fused_state, three_state.double(), 1e-6, "states, fused against three kernels")
+    assert (fused[5:] == 0).all()
+    for slot in (2, 6):
+        assert torch.equal(fused_state[slot].transpose(-1, -2).cpu(), state[slot])
 
 
 def test_delta_rule_token_by_token_is_the_prompt_bit_for_bit():
@@ -156,7 +190,7 @@ def test_delta_rule_token_by_token_is_the_prompt_bit_for_bit():
         assert torch.equal(rows, results[0][0]) and torch.equal(st, results[0][1])
     want_raw, want, final = delta_plain(packed, t, H, D, rank, eps, torch.zeros(H, D, D))
     close(results[0][0], want, 8e-3, "300 tokens")
-    close(results[0][1], final, 2e-5, "state after 300 tokens")
+    close(results[0][1].transpose(-1, -2), final, 2e-5, "state after 300 tokens")
 
 
 def test_delta_rule_full_removal_replaces_a_key():
