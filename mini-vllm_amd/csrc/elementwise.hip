@@ -896,37 +896,86 @@ extern "C" int mv_swiglu(const void* gate_up, void* out, int n, int I, int dtype
 //   out[r] = v / sqrt(mean(v^2) + eps_b) * wb                          (out == null: the add alone)
 // One workgroup per row; the sum stays float from the first norm to the second.
 // ---------------------------------------------------------------------------------------
-template <typename T>
+// NE > 0: a thread keeps its NE columns (c = thread + 256 e) in registers from the first sum to the last
+// store, so y and the residual are read once (rows of up to 256 NE columns); NE = 0: rows of any length,
+// read again for every pass.
+template <typename T, int NE>
 __global__ void __launch_bounds__(256)
 norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_a, int unit_a, float* __restrict__ resid,
                      WeightPtr wb, float eps_b, int unit_b, T* __restrict__ out, int h) {
-    __shared__ float scratch[17];
+    __shared__ float part_a[4], part_b[4];
     const int r = blockIdx.x;
+    const int lane = threadIdx.x % MV_WAVE, wave = threadIdx.x / MV_WAVE;
     const T* yr = y + (size_t)r * ldy;
     float* x = resid + (size_t)r * h;
-    float ss = 0.f;
-    for (int c = threadIdx.x; c < h; c += blockDim.x) {
-        const float v = to_f(yr[c]);
-        ss = fmaf(v, v, ss);
-    }
-    ss = block_sum(ss, scratch);
-    const float ra = 1.f / sqrtf(ss / (float)h + eps_a);
-    float ss2 = 0.f;
-    for (int c = threadIdx.x; c < h; c += blockDim.x) {
-        float w = wa.at(c);
-        if (unit_a) w += 1.f;
-        const float v = x[c] + to_f(yr[c]) * ra * w;
-        x[c] = v;
-        ss2 = fmaf(v, v, ss2);
-    }
-    if (out == nullptr) return;
-    ss2 = block_sum(ss2, scratch);
-    const float rb = 1.f / sqrtf(ss2 / (float)h + eps_b);
-    T* o = out + (size_t)r * h;
-    for (int c = threadIdx.x; c < h; c += blockDim.x) {
-        float w = wb.at(c);
-        if (unit_b) w += 1.f;
-        o[c] = from_f<T>(x[c] * rb * w);      // the thread's own store of x[c] above
+    T* o = out ? out + (size_t)r * h : nullptr;
+    if constexpr (NE > 0) {
+        float v[NE];
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            const int c = threadIdx.x + 256 * e;
+            v[e] = c < h ? to_f(yr[c]) : 0.f;
+            ss = fmaf(v[e], v[e], ss);
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) part_a[wave] = ss;
+        __syncthreads();
+        const float ra = 1.f / sqrtf((part_a[0] + part_a[1] + part_a[2] + part_a[3]) / (float)h + eps_a);
+        float ss2 = 0.f;
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            const int c = threadIdx.x + 256 * e;
+            if (c < h) {
+                float w = wa.at(c);
+                if (unit_a) w += 1.f;
+                v[e] = x[c] + v[e] * ra * w;
+                x[c] = v[e];
+                ss2 = fmaf(v[e], v[e], ss2);
+            }
+        }
+        if (o == nullptr) return;
+        ss2 = wave_sum(ss2);
+        if (lane == 0) part_b[wave] = ss2;
+        __syncthreads();
+        const float rb = 1.f / sqrtf((part_b[0] + part_b[1] + part_b[2] + part_b[3]) / (float)h + eps_b);
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            const int c = threadIdx.x + 256 * e;
+            if (c < h) {
+                float w = wb.at(c);
+                if (unit_b) w += 1.f;
+                o[c] = from_f<T>(v[e] * rb * w);
+            }
+        }
+    } else {
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < h; c += 256) {
+            const float v = to_f(yr[c]);
+            ss = fmaf(v, v, ss);
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) part_a[wave] = ss;
+        __syncthreads();
+        const float ra = 1.f / sqrtf((part_a[0] + part_a[1] + part_a[2] + part_a[3]) / (float)h + eps_a);
+        float ss2 = 0.f;
+        for (int c = threadIdx.x; c < h; c += 256) {
+            float w = wa.at(c);
+            if (unit_a) w += 1.f;
+            const float v = x[c] + to_f(yr[c]) * ra * w;
+            x[c] = v;
+            ss2 = fmaf(v, v, ss2);
+        }
+        if (o == nullptr) return;
+        ss2 = wave_sum(ss2);
+        if (lane == 0) part_b[wave] = ss2;
+        __syncthreads();
+        const float rb = 1.f / sqrtf((part_b[0] + part_b[1] + part_b[2] + part_b[3]) / (float)h + eps_b);
+        for (int c = threadIdx.x; c < h; c += 256) {
+            float w = wb.at(c);
+            if (unit_b) w += 1.f;
+            o[c] = from_f<T>(x[c] * rb * w);      // the thread's own store of x[c] above
+        }
     }
 }
 
@@ -938,9 +987,20 @@ extern "C" int mv_norm_add_norm(const void* y, long ldy, const void* wa, int wa_
     MV_REQUIRE(out == nullptr || (wb && mv_valid_dtype(wb_dtype) && eps_b > 0.f), "norm_add_norm: the second norm lacks its weight");
     if (n == 0) return 0;
     WeightPtr pa{wa, wa_dtype}, pb{wb, out ? wb_dtype : MV_F32};
-    MV_DISPATCH_T(dtype, "norm_add_norm",
-                  hipLaunchKernelGGL(norm_add_norm_kernel<T>, dim3(n), dim3(256), 0, stream, (const T*)y, ldy, pa, eps_a,
-                                     unit_a, resid, pb, eps_b, unit_b, (T*)out, h));
+#define NAN_LAUNCH(NE)                                                                                               \
+    MV_DISPATCH_T(dtype, "norm_add_norm",                                                                            \
+                  hipLaunchKernelGGL((norm_add_norm_kernel<T, NE>), dim3(n), dim3(256), 0, stream, (const T*)y, ldy, pa, \
+                                     eps_a, unit_a, resid, pb, eps_b, unit_b, (T*)out, h))
+    if (h <= 1024) {
+        NAN_LAUNCH(4);
+    } else if (h <= 4096) {
+        NAN_LAUNCH(16);
+    } else if (h <= 8192) {
+        NAN_LAUNCH(32);
+    } else {
+        NAN_LAUNCH(0);
+    }
+#undef NAN_LAUNCH
     return mv_check_launch("norm_add_norm");
 }
 

@@ -82,6 +82,28 @@ extern "C" int mv_token_shift(const void* h, long ldh, void* out, long ldo, cons
 
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
 
+// NT sums over j in [j0, j1) of w2t[j][c] * th[t][j] (th rows `pitch` floats apart), the weight's element
+// type known at compile time and eight loads in flight at a time; the additions run in the order of j
+template <typename W, int NT>
+__device__ __forceinline__ void decay_dots(const W* __restrict__ w2t_c, size_t inner, const float* th, int pitch, int j0,
+                                           int j1, float (&acc)[NT]) {
+    int j = j0;
+    for (; j + 8 <= j1; j += 8) {
+        float w[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) w[e] = to_f(w2t_c[(size_t)(j + e) * inner]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[t] = fmaf(w[e], th[t * pitch + j + e], acc[t]);
+    }
+    for (; j < j1; ++j) {
+        const float w = to_f(w2t_c[(size_t)j * inner]);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = fmaf(w, th[t * pitch + j], acc[t]);
+    }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 delta_prepare_kernel(const T* __restrict__ packed, long ld, int H, int D, int rank, WeightPtr w2t, WeightPtr w0,
@@ -119,11 +141,10 @@ delta_prepare_kernel(const T* __restrict__ packed, long ld, int H, int D, int ra
     float acc[DP_TOKENS];
 #pragma unroll
     for (int tt = 0; tt < DP_TOKENS; ++tt) acc[tt] = 0.f;
-    for (int j = 0; j < rank; ++j) {
-        const float w = w2t.at((size_t)j * inner + c);
-#pragma unroll
-        for (int tt = 0; tt < DP_TOKENS; ++tt) acc[tt] = fmaf(w, th[tt][j], acc[tt]);
-    }
+    if (w2t.dtype == MV_F32)
+        decay_dots<float, DP_TOKENS>((const float*)w2t.p + c, inner, &th[0][0], DP_MAX_RANK, 0, rank, acc);
+    else
+        decay_dots<bf16, DP_TOKENS>((const bf16*)w2t.p + c, inner, &th[0][0], DP_MAX_RANK, 0, rank, acc);
     const float b0 = w0.at(c), ab = a_bias.at(c);
     const int head = c / D, d = c % D;
     const int hh = head - h_lo;
@@ -338,9 +359,11 @@ delta_scan_kernel(const T* __restrict__ packed, long ld, const float* __restrict
 
 // how a head of size D is dealt out: (rows a lane keeps, lanes a column); 0 when D is not served
 static void delta_scan_shape(int D, int& R, int& L) {
+    // few rows a lane and many lanes a column: a token costs the fewest instructions of the one wave a
+    // SIMD runs, and a head is spread over the most workgroups
     if (D <= 16) { R = 4; L = 4; }
-    else if (D <= 32) { R = 8; L = 4; }
-    else if (D <= 64) { R = 8; L = 8; }
+    else if (D <= 32) { R = 4; L = 8; }
+    else if (D <= 64) { R = 4; L = 16; }
     else if (D <= 128) { R = 8; L = 16; }
     else { R = 16; L = 16; }
 }
@@ -364,10 +387,10 @@ extern "C" int mv_delta_scan(const void* packed, long ld, const float* coef, flo
                                      state, cu_seqlens, state_slots, H, D, out, n))
     if (R == 4 && L == 4) {
         DS_LAUNCH(4, 4);
-    } else if (R == 8 && L == 4) {
-        DS_LAUNCH(8, 4);
-    } else if (R == 8 && L == 8) {
-        DS_LAUNCH(8, 8);
+    } else if (R == 4 && L == 8) {
+        DS_LAUNCH(4, 8);
+    } else if (R == 4 && L == 16) {
+        DS_LAUNCH(4, 16);
     } else if (R == 8 && L == 16) {
         DS_LAUNCH(8, 16);
     } else {
@@ -396,6 +419,7 @@ delta_step_kernel(const T* __restrict__ packed, long ld, int H, int D, int rank,
     __shared__ __attribute__((aligned(16))) float vec[5][DPAD];
     __shared__ float vals[DPAD];
     __shared__ float outs[DPAD];
+    __shared__ float partial[256];               // [parts][D], parts * D <= 256
     __shared__ float red[8];
     const int t = blockIdx.x, head = blockIdx.y;
     const int tid = threadIdx.x;
@@ -420,12 +444,31 @@ delta_step_kernel(const T* __restrict__ packed, long ld, int H, int D, int rank,
         if (lane == 0) red[0] = 1.f / sqrtf(ss + key_eps);
     }
     __syncthreads();
+    // the decay's small product, dealt out over all threads: thread (part, d) sums a run of j for channel d
+    // (one part when D >= 256), the parts are added in order
+    {
+        const int parts = D >= 256 ? 1 : 256 / D;
+        const int per = (rank + parts - 1) / parts;
+        for (int x = tid; x < parts * D; x += 256) {
+            const int part = x / D, d = x % D;
+            const int cc = head * D + d;
+            const int j0 = min(rank, part * per), j1 = min(rank, j0 + per);
+            float acc[1] = {0.f};
+            if (w2t.dtype == MV_F32)
+                decay_dots<float, 1>((const float*)w2t.p + cc, inner, th, 0, j0, j1, acc);
+            else
+                decay_dots<bf16, 1>((const bf16*)w2t.p + cc, inner, th, 0, j0, j1, acc);
+            partial[part * D + d] = acc[0];
+        }
+    }
+    __syncthreads();
     for (int d = tid; d < DPAD; d += 256) {
         float w = 0.f, au = 0.f, u = 0.f, k = 0.f, r = 0.f, v = 0.f;
         if (d < D) {
             const int cc = head * D + d;
+            const int parts = D >= 256 ? 1 : 256 / D;
             float acc = 0.f;
-            for (int j = 0; j < rank; ++j) acc = fmaf(w2t.at((size_t)j * inner + cc), th[j], acc);
+            for (int part = 0; part < parts; ++part) acc += partial[part * D + d];
             k = to_f(p[inner + cc]);
             u = k * red[0];
             au = sigmoid_f(to_f(p[4 * (size_t)inner + cc]) + a_bias.at(cc)) * u;
@@ -488,10 +531,10 @@ extern "C" int mv_delta_step(const void* packed, long ld, int n, int H, int D, i
                                      (T*)out, ldo))
     if (R == 4 && L == 4) {
         DT_LAUNCH(4, 4);
-    } else if (R == 8 && L == 4) {
-        DT_LAUNCH(8, 4);
-    } else if (R == 8 && L == 8) {
-        DT_LAUNCH(8, 8);
+    } else if (R == 4 && L == 8) {
+        DT_LAUNCH(4, 8);
+    } else if (R == 4 && L == 16) {
+        DT_LAUNCH(4, 16);
     } else if (R == 8 && L == 16) {
         DT_LAUNCH(8, 16);
     } else {
