@@ -897,25 +897,59 @@ extern "C" int mv_swiglu(const void* gate_up, void* out, int n, int I, int dtype
 // One workgroup per row; the sum stays float from the first norm to the second.
 // ---------------------------------------------------------------------------------------
 // NE > 0: a thread keeps its NE columns (c = thread + 256 e) in registers from the first sum to the last
-// store, so y and the residual are read once (rows of up to 256 NE columns); NE = 0: rows of any length,
-// read again for every pass.
+// store, and everything it needs from memory is asked for before the first sum, so the kernel waits for
+// memory once (rows of up to 256 NE columns); NE = 0: rows of any length, read again for every pass.
+//
+// With a token shift (steps in which every request brings one token): row r belongs to request
+// token_seq[r]; what goes to `out` is h + (prev - h) * mix with h the normalised row as it is stored
+// (rounded to T) and prev the request's row of `shift_state`, which then takes h. A padding row
+// (token_seq < 0) gives zeros and touches no state.
+struct ShiftArgs {
+    const void* mix;           // null: no shift
+    int mix_dtype;
+    void* state;               // [slots][h] of T
+    const int* token_seq;
+    const int* state_slots;
+};
+
 template <typename T, int NE>
 __global__ void __launch_bounds__(256)
 norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_a, int unit_a, float* __restrict__ resid,
-                     WeightPtr wb, float eps_b, int unit_b, T* __restrict__ out, int h) {
+                     WeightPtr wb, float eps_b, int unit_b, T* __restrict__ out, int h, ShiftArgs shift) {
     __shared__ float part_a[4], part_b[4];
     const int r = blockIdx.x;
     const int lane = threadIdx.x % MV_WAVE, wave = threadIdx.x / MV_WAVE;
     const T* yr = y + (size_t)r * ldy;
     float* x = resid + (size_t)r * h;
     T* o = out ? out + (size_t)r * h : nullptr;
+    const bool shifted = shift.mix != nullptr && o != nullptr;
+    const int seq = shifted ? shift.token_seq[r] : 0;
+    T* st = (shifted && seq >= 0) ? (T*)shift.state + (size_t)shift.state_slots[seq] * h : nullptr;
+    const WeightPtr mix{shift.mix, shift.mix_dtype};
+    auto finish = [&](int c, float normed) {
+        // the row as it is stored, then (with a shift) mixed with the request's row before it
+        const T hT = from_f<T>(normed);
+        if (!shifted) {
+            o[c] = hT;
+        } else if (st == nullptr) {
+            o[c] = from_f<T>(0.f);
+        } else {
+            const float hf = to_f(hT), prev = to_f(st[c]);
+            st[c] = hT;
+            o[c] = from_f<T>(hf + (prev - hf) * mix.at(c));
+        }
+    };
     if constexpr (NE > 0) {
-        float v[NE];
+        float v[NE], xr[NE], fa[NE], fb[NE];
         float ss = 0.f;
 #pragma unroll
         for (int e = 0; e < NE; ++e) {
             const int c = threadIdx.x + 256 * e;
-            v[e] = c < h ? to_f(yr[c]) : 0.f;
+            const bool ok = c < h;
+            v[e] = ok ? to_f(yr[c]) : 0.f;
+            xr[e] = ok ? x[c] : 0.f;
+            fa[e] = ok ? wa.at(c) + (unit_a ? 1.f : 0.f) : 0.f;
+            fb[e] = (ok && o != nullptr) ? wb.at(c) + (unit_b ? 1.f : 0.f) : 0.f;
             ss = fmaf(v[e], v[e], ss);
         }
         ss = wave_sum(ss);
@@ -927,9 +961,7 @@ norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_
         for (int e = 0; e < NE; ++e) {
             const int c = threadIdx.x + 256 * e;
             if (c < h) {
-                float w = wa.at(c);
-                if (unit_a) w += 1.f;
-                v[e] = x[c] + v[e] * ra * w;
+                v[e] = xr[e] + v[e] * ra * fa[e];
                 x[c] = v[e];
                 ss2 = fmaf(v[e], v[e], ss2);
             }
@@ -942,11 +974,7 @@ norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_
 #pragma unroll
         for (int e = 0; e < NE; ++e) {
             const int c = threadIdx.x + 256 * e;
-            if (c < h) {
-                float w = wb.at(c);
-                if (unit_b) w += 1.f;
-                o[c] = from_f<T>(v[e] * rb * w);
-            }
+            if (c < h) finish(c, v[e] * rb * fb[e]);
         }
     } else {
         float ss = 0.f;
@@ -974,14 +1002,18 @@ norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_
         for (int c = threadIdx.x; c < h; c += 256) {
             float w = wb.at(c);
             if (unit_b) w += 1.f;
-            o[c] = from_f<T>(x[c] * rb * w);      // the thread's own store of x[c] above
+            finish(c, x[c] * rb * w);             // the thread's own store of x[c] above
         }
     }
 }
 
 extern "C" int mv_norm_add_norm(const void* y, long ldy, const void* wa, int wa_dtype, float eps_a, int unit_a,
                                 float* resid, const void* wb, int wb_dtype, float eps_b, int unit_b, void* out, int n,
-                                int h, int dtype, hipStream_t stream) {
+                                int h, const void* shift_mix, int shift_mix_dtype, void* shift_state,
+                                const int* token_seq, const int* state_slots, int dtype, hipStream_t stream) {
+    MV_REQUIRE(shift_mix == nullptr || (out && shift_state && token_seq && state_slots && mv_valid_dtype(shift_mix_dtype)),
+               "norm_add_norm: a token shift needs its state, the rows' requests, their slots and an output");
+    const ShiftArgs shift{shift_mix, shift_mix_dtype, shift_state, token_seq, state_slots};
     MV_REQUIRE(n >= 0 && h > 0 && ldy >= h, "norm_add_norm: bad sizes n=%d h=%d", n, h);
     MV_REQUIRE(y && wa && resid && mv_valid_dtype(wa_dtype) && eps_a > 0.f, "norm_add_norm: missing operand");
     MV_REQUIRE(out == nullptr || (wb && mv_valid_dtype(wb_dtype) && eps_b > 0.f), "norm_add_norm: the second norm lacks its weight");
@@ -990,7 +1022,7 @@ extern "C" int mv_norm_add_norm(const void* y, long ldy, const void* wa, int wa_
 #define NAN_LAUNCH(NE)                                                                                               \
     MV_DISPATCH_T(dtype, "norm_add_norm",                                                                            \
                   hipLaunchKernelGGL((norm_add_norm_kernel<T, NE>), dim3(n), dim3(256), 0, stream, (const T*)y, ldy, pa, \
-                                     eps_a, unit_a, resid, pb, eps_b, unit_b, (T*)out, h))
+                                     eps_a, unit_a, resid, pb, eps_b, unit_b, (T*)out, h, shift))
     if (h <= 1024) {
         NAN_LAUNCH(4);
     } else if (h <= 4096) {

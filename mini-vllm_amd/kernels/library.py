@@ -66,9 +66,11 @@ _SIGNATURES = {
     "mv_attention_sigmoid_ref": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                          c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
                                          c_void_p, c_void_p, c_long, c_int, c_void_p]),
-    # y, ldy, wa, wa_dtype, eps_a, unit_a, resid, wb, wb_dtype, eps_b, unit_b, out, n, h, dtype, stream
+    # y, ldy, wa, wa_dtype, eps_a, unit_a, resid, wb, wb_dtype, eps_b, unit_b, out, n, h, shift_mix, shift_mix_dtype,
+    # shift_state, token_seq, state_slots, dtype, stream
     "mv_norm_add_norm": (c_int, [c_void_p, c_long, c_void_p, c_int, c_float, c_int, c_void_p, c_void_p, c_int, c_float,
-                                 c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
+                                 c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                 c_void_p]),
     # x, ld, rows, cols, cap, stream
     "mv_soft_cap": (c_int, [c_void_p, c_long, c_int, c_int, c_float, c_void_p]),
     "mv_sample": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

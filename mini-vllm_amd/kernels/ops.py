@@ -559,9 +559,14 @@ class Ops:
                       weight.data_ptr(), _weight_code(weight, "delta norm weight"), n, heads, dim, float(eps),
                       out.data_ptr(), out.stride(0) if n > 1 else inner, self.code, self._stream())
 
-    def norm_add_norm(self, y: torch.Tensor, norm_y, resid: torch.Tensor, norm_next, out: Optional[torch.Tensor]) -> None:
+    def norm_add_norm(self, y: torch.Tensor, norm_y, resid: torch.Tensor, norm_next, out: Optional[torch.Tensor],
+                      shift: Optional[tuple] = None) -> None:
         """resid += rmsnorm(y) * w (``norm_y`` = (weight, eps, unit_offset)); with ``norm_next`` of the same
-        form, out = rmsnorm(resid) * w'. The sum stays float32 in between."""
+        form, out = rmsnorm(resid) * w'. The sum stays float32 in between.
+
+        ``shift`` = (mix, state [slots, h], token_seq, state_slots), for steps in which every request brings
+        one token: ``out`` gets the rows after the token shift that ``token_shift`` would apply to them (row r
+        belongs to request token_seq[r]; the state takes the unshifted row)."""
         self._act(y, "sublayer output"); _dev(resid, "residual")
         n, h = resid.shape
         if resid.dtype != torch.float32 or not resid.is_contiguous() or tuple(y.shape) != (n, h) or y.stride(1) != 1:
@@ -580,10 +585,22 @@ class Ops:
             wb_code = _weight_code(wb, "norm weight")
             if wb.numel() != h or not wb.is_contiguous() or tuple(out.shape) != (n, h) or not out.is_contiguous():
                 raise KernelLibraryError("norm_add_norm: the second norm's weight or output does not fit")
-        self._note("mv_norm_add_norm", self._size(y, out) + 2 * self._size(resid), 8 * n * h)
+        mix = state = tsq = slots = None
+        mix_code = DTYPE_F32
+        if shift is not None:
+            mix, state, tsq, slots = shift
+            if out is None:
+                raise KernelLibraryError("norm_add_norm: a token shift needs the second norm and its output")
+            self._act(state, "shift state"); _dev(mix, "shift weight")
+            mix_code = _weight_code(mix, "shift weight")
+            if state.dim() != 2 or state.shape[1] != h or not state.is_contiguous() or mix.numel() != h or not mix.is_contiguous():
+                raise KernelLibraryError(f"norm_add_norm: shift state {tuple(state.shape)} / weight do not fit rows of {h}")
+            self._ints(n, token_seq=(tsq, n), state_slots=(slots, 1))
+        self._note("mv_norm_add_norm", self._size(y, out) + 2 * self._size(resid) + (2 * self._size(out) if shift else 0), 8 * n * h)
         self.lib.call("mv_norm_add_norm", y.data_ptr(), y.stride(0) if n > 1 else h, wa.data_ptr(),
                       _weight_code(wa, "norm weight"), float(eps_a), int(unit_a), resid.data_ptr(), _ptr(wb), wb_code,
-                      float(eps_b), int(unit_b), _ptr(out), n, h, self.code, self._stream())
+                      float(eps_b), int(unit_b), _ptr(out), n, h, _ptr(mix), mix_code, _ptr(state), _ptr(tsq), _ptr(slots),
+                      self.code, self._stream())
 
     def soft_cap(self, logits: torch.Tensor, cap: float) -> None:
         """In place on float32 [rows, cols]: x <- cap * tanh(x / cap)."""

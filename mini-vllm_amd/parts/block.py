@@ -117,24 +117,30 @@ class SandwichBlock(Block):
         return self.norm_in
 
     def entry_part(self):
-        return None            # the rows pass through the shift first: no product takes the norm over
+        # the rows pass through the shift first: no product takes the norm over; a block in front may
+        # apply this block's shift together with its norm (``TokenShiftEntry``)
+        return TokenShiftEntry(self.shift) if self.shift is not None else None
 
     def forward(self, stream: HiddenStream, ctx, call: int, next_norm: Optional[Norm] = None, next_part=None) -> None:
+        already = stream.normed is not None and len(stream.normed) > 2 and stream.normed[2] is self.shift
         h = self.norm_in.forward(stream, ctx)
-        if self.shift is not None:
+        if self.shift is not None and not already:
             mixed = self.rt.workspace.get("shift.out", tuple(h.shape), h.dtype)
             self.rt.ops.token_shift(h, self.shift, ctx.state(call, "shift.last"), ctx.token_seq, ctx.cu_seqlens,
                                     ctx.state_slots, mixed)
             h = mixed
         y = self.mixer.forward(h, ctx, call)
-        self._close(stream, ctx, y, self.norm_out, self.norm_ffn_in if self.ffn is not None else next_norm)
-        if self.ffn is not None:
+        last = self.ffn is None
+        self._close(stream, ctx, y, self.norm_out, next_norm if last else self.norm_ffn_in, call, next_part if last else None)
+        if not last:
             h = self.norm_ffn_in.forward(stream, ctx)
             y = self.ffn.forward(h, ctx)
-            self._close(stream, ctx, y, self.norm_ffn_out, next_norm)
+            self._close(stream, ctx, y, self.norm_ffn_out, next_norm, call, next_part)
 
-    def _close(self, stream: HiddenStream, ctx, y, norm_out: Norm, norm_next: Optional[Norm]) -> None:
-        """resid += norm_out(y); the rows of ``norm_next`` are left in the stream when it can ride along."""
+    def _close(self, stream: HiddenStream, ctx, y, norm_out: Norm, norm_next: Optional[Norm], call: int = 0,
+               next_part=None) -> None:
+        """resid += norm_out(y); the rows of ``norm_next`` are left in the stream when it can ride along, and
+        in a step of single tokens the next block's token shift with them."""
         if not isinstance(y, torch.Tensor):
             y = y.materialize()
         out_form = norm_out.as_scaled_rms()
@@ -147,6 +153,22 @@ class SandwichBlock(Block):
         rows = None
         if next_form is not None:
             rows = self.rt.workspace.get("normed", tuple(y.shape), y.dtype)
-        self.rt.ops.norm_add_norm(y, out_form, stream.resid, next_form, rows)
+        shift = None
+        plan = getattr(ctx, "attention_plan", None)
+        if rows is not None and isinstance(next_part, TokenShiftEntry) and plan is not None and plan.decode_only:
+            # the block that runs next is call + 1: its shift state is that call's
+            shift = (next_part.mix, ctx.state(call + 1, "shift.last"), ctx.token_seq, ctx.state_slots)
+        self.rt.ops.norm_add_norm(y, out_form, stream.resid, next_form, rows, shift=shift)
         stream.delta = None
-        stream.normed = (norm_next, rows) if rows is not None else None
+        if rows is None:
+            stream.normed = None
+        else:
+            stream.normed = (norm_next, rows, next_part.mix) if shift is not None else (norm_next, rows)
+
+
+class TokenShiftEntry:
+    """What a sandwich block with a token shift offers the block in front of it: the shift's weights, so
+    that its rows can leave that block's last kernel already shifted."""
+
+    def __init__(self, mix: torch.Tensor):
+        self.mix = mix

@@ -369,6 +369,37 @@ def test_norms_around_a_sublayer(dtype, h):
     assert torch.equal(r2, r)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("h", [48, 1024, 5000, 9000])
+def test_norms_with_the_next_token_shift(dtype, h):
+    """A step of single tokens: the kernel that closes a sublayer also applies the next layer's token
+    shift. The same bits as the two kernels it stands for; a padding row touches no state."""
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(h)
+    n, slots = 5, [2, 0, 3, 1]
+    y = (torch.randn(n, h, generator=g) * 3).to(dtype).to(DEV)
+    resid = torch.randn(n, h, generator=g).to(DEV)
+    wa = (1 + 0.1 * torch.randn(h, generator=g)).to(torch.bfloat16).to(DEV)
+    wb = (1 + 0.1 * torch.randn(h, generator=g)).to(torch.bfloat16).to(DEV)
+    mix = torch.rand(h, generator=g).to(torch.bfloat16).to(DEV)
+    state = torch.randn(5, h, generator=g).to(dtype).to(DEV)
+    tsq, cu, sl = step_ints([1, 1, 1, 1], slots, pad_rows=1)
+    r1, s1 = resid.clone(), state.clone()
+    rows = torch.empty(n, h, dtype=dtype, device=DEV)
+    want = torch.empty(n, h, dtype=dtype, device=DEV)
+    ops.norm_add_norm(y, (wa, 1e-5, False), r1, (wb, 2e-6, False), rows)
+    ops.token_shift(rows, mix, s1, tsq, cu, sl, want)
+    r2, s2 = resid.clone(), state.clone()
+    got = torch.empty(n, h, dtype=dtype, device=DEV)
+    ops.norm_add_norm(y, (wa, 1e-5, False), r2, (wb, 2e-6, False), got, shift=(mix, s2, tsq, sl))
+    torch.cuda.synchronize()
+    assert torch.equal(r1, r2) and torch.equal(s1, s2) and torch.equal(got, want)
+    assert torch.equal(s2[4], state[4]) and (got[4] == 0).all()
+    prev = state[slots[1]].double().cpu()
+    hrow = rows[1].double().cpu()
+    close(got[1], hrow + (prev - hrow) * mix.double().cpu(), 1e-6 if dtype == torch.float32 else 8e-3)
+
+
 def test_soft_cap():
     ops = ops_for(torch.float32)
     x = torch.linspace(-90, 90, 7 * 333).view(7, 333)
