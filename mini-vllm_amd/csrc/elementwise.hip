@@ -940,12 +940,13 @@ norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_
         }
     };
     if constexpr (NE > 0) {
-        float v[NE], xr[NE], fa[NE], fb[NE];
+        float v[NE], xr[NE], fa[NE], fb[NE], prev[NE];
         float ss = 0.f;
 #pragma unroll
         for (int e = 0; e < NE; ++e) {
             const int c = threadIdx.x + 256 * e;
             const bool ok = c < h;
+            prev[e] = (ok && st != nullptr) ? to_f(st[c]) : 0.f;      // (only this thread ever touches st[c])
             v[e] = ok ? to_f(yr[c]) : 0.f;
             xr[e] = ok ? x[c] : 0.f;
             fa[e] = ok ? wa.at(c) + (unit_a ? 1.f : 0.f) : 0.f;
@@ -974,7 +975,15 @@ norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_
 #pragma unroll
         for (int e = 0; e < NE; ++e) {
             const int c = threadIdx.x + 256 * e;
-            if (c < h) finish(c, v[e] * rb * fb[e]);
+            if (c >= h) continue;
+            if (st == nullptr) {
+                finish(c, v[e] * rb * fb[e]);
+            } else {
+                const T hT = from_f<T>(v[e] * rb * fb[e]);
+                const float hf = to_f(hT);
+                st[c] = hT;
+                o[c] = from_f<T>(hf + (prev[e] - hf) * mix.at(c));
+            }
         }
     } else {
         float ss = 0.f;
