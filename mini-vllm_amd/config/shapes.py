@@ -25,7 +25,12 @@ def named_shapes() -> Dict[str, Dict[str, Any]]:
     """Every named shape as a raw config.json dictionary, ``architectures`` included: the registry
     picks the architecture from it, as it does for a model folder. Another architecture's shapes are
     added here."""
-    return {name: qwen3_shape(name) for name in QWEN3_SHAPES}
+    shapes = {name: qwen3_shape(name) for name in QWEN3_SHAPES}
+    shapes["bolapel-tiny"] = bolapel_tiny_shape()
+    for name in QWEN3_SHAPES:
+        if name != "tiny":
+            shapes[f"bolapel-{name}"] = bolapel_shape(name)
+    return shapes
 
 
 def named_shape(name: str, **overrides) -> Dict[str, Any]:
@@ -70,3 +75,16 @@ def bolapel_shape(name: str, layers: int = None, chunk: int = 1024, delta_head_d
                         "mixer": {"heads": hid // delta_head_dim, "dim": delta_head_dim, "rank": decay_rank}})
     return {"architecture": "Bolapel", "vocab": q["vocab_size"], "width": hid, "layers": out,
             "norm": {"eps": q["rms_norm_eps"]}, "logit_softcap": 30.0}
+
+
+def bolapel_tiny_shape() -> Dict[str, Any]:
+    """A Bolapel model of a few thousand weights with every kind of layer: delta rule, attention in chunks
+    with keys of its own, a layer without feed-forward, attention on another layer's keys."""
+    ff = {"kind": "dense", "ff": 96}
+    attn = {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.25, "mask": {"size": 24},
+            "rot": {"dims": 8, "base": 10000.0}}
+    return {"architecture": "Bolapel", "vocab": 256, "width": 64, "norm": {"eps": 1e-5}, "logit_softcap": 20.0,
+            "layers": [{"type": "general_delta", "mixer": {"heads": 2, "dim": 16, "rank": 8}, "mlp": ff},
+                       {"type": "attention", "mixer": dict(attn), "mlp": ff},
+                       {"type": "general_delta", "mixer": {"heads": 4, "dim": 8, "rank": 8}, "mlp": None},
+                       {"type": "attention", "mixer": dict(attn, kv_from=1), "mlp": ff}]}

@@ -942,15 +942,22 @@ norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_
     if constexpr (NE > 0) {
         float v[NE], xr[NE], fa[NE], fb[NE], prev[NE];
         float ss = 0.f;
+        // every load is issued whatever the column (beyond the row's end the last column is read again and
+        // the value dropped): a load under a condition would be a branch with a wait of its own, and the
+        // kernel would wait for memory once per column instead of once
+        const T* stl = st != nullptr ? st : yr;
+        const WeightPtr wbl = o != nullptr ? wb : wa;
 #pragma unroll
         for (int e = 0; e < NE; ++e) {
             const int c = threadIdx.x + 256 * e;
             const bool ok = c < h;
-            prev[e] = (ok && st != nullptr) ? to_f(st[c]) : 0.f;      // (only this thread ever touches st[c])
-            v[e] = ok ? to_f(yr[c]) : 0.f;
-            xr[e] = ok ? x[c] : 0.f;
-            fa[e] = ok ? wa.at(c) + (unit_a ? 1.f : 0.f) : 0.f;
-            fb[e] = (ok && o != nullptr) ? wb.at(c) + (unit_b ? 1.f : 0.f) : 0.f;
+            const int cl = ok ? c : h - 1;
+            const float l_prev = to_f(stl[cl]), l_y = to_f(yr[cl]), l_x = x[cl], l_a = wa.at(cl), l_b = wbl.at(cl);
+            prev[e] = l_prev;                                          // (st[c] is written by this thread only, below)
+            v[e] = ok ? l_y : 0.f;
+            xr[e] = l_x;
+            fa[e] = l_a + (unit_a ? 1.f : 0.f);
+            fb[e] = l_b + (unit_b ? 1.f : 0.f);
             ss = fmaf(v[e], v[e], ss);
         }
         ss = wave_sum(ss);

@@ -148,20 +148,29 @@ delta_prepare_kernel(const T* __restrict__ packed, long ld, int H, int D, int ra
     const float b0 = w0.at(c), ab = a_bias.at(c);
     const int head = c / D, d = c % D;
     const int hh = head - h_lo;
+    // (the rows' loads first, all of them, from clamped rows: under a condition each would wait on its own)
+    float lk[DP_TOKENS], la[DP_TOKENS], lr[DP_TOKENS];
 #pragma unroll
     for (int tt = 0; tt < DP_TOKENS; ++tt) {
-        if (tt >= nt) break;
-        const size_t row = (size_t)(t0 + tt);
-        const T* p = packed + row * ld;
-        const float k = to_f(p[inner + c]);
-        const float u = k * inv_len[tt][hh];
-        const float rate = sigmoid_f(to_f(p[4 * (size_t)inner + c]) + ab);
-        float* o = coef + ((row * H + head) * 5) * (size_t)D + d;
-        o[0] = expf(-decay_rate * sigmoid_f(acc[tt] + b0));
-        o[D] = rate * u;
-        o[2 * D] = u;
-        o[3 * D] = k;
-        o[4 * D] = to_f(p[c]);
+        const T* p = packed + (size_t)(t0 + (tt < nt ? tt : 0)) * ld;
+        lk[tt] = to_f(p[inner + c]);
+        la[tt] = to_f(p[4 * (size_t)inner + c]);
+        lr[tt] = to_f(p[c]);
+    }
+#pragma unroll
+    for (int tt = 0; tt < DP_TOKENS; ++tt) {
+        if (tt < nt) {
+            const size_t row = (size_t)(t0 + tt);
+            const float k = lk[tt];
+            const float u = k * inv_len[tt][hh];
+            const float rate = sigmoid_f(la[tt] + ab);
+            float* o = coef + ((row * H + head) * 5) * (size_t)D + d;
+            o[0] = expf(-decay_rate * sigmoid_f(acc[tt] + b0));
+            o[D] = rate * u;
+            o[2 * D] = u;
+            o[3 * D] = k;
+            o[4 * D] = lr[tt];
+        }
     }
 }
 
@@ -252,13 +261,13 @@ __device__ __forceinline__ void delta_state_io(float (&s)[R], float* column, int
     if ((D & 3) == 0) {
 #pragma unroll
         for (int e = 0; e < R; e += 4) {
-            float4* p = reinterpret_cast<float4*>(column + i0 + e);
             const bool ok = live && i0 + e < D;
+            float4* p = reinterpret_cast<float4*>(column + (i0 + e < D ? i0 + e : 0));
             if constexpr (STORE) {
                 if (ok) *p = float4{s[e], s[e + 1], s[e + 2], s[e + 3]};
             } else {
-                const float4 v = ok ? *p : float4{0.f, 0.f, 0.f, 0.f};
-                s[e] = v.x; s[e + 1] = v.y; s[e + 2] = v.z; s[e + 3] = v.w;
+                const float4 v = *p;                  // always issued (a valid address either way), dropped where it does not count
+                s[e] = ok ? v.x : 0.f; s[e + 1] = ok ? v.y : 0.f; s[e + 2] = ok ? v.z : 0.f; s[e + 3] = ok ? v.w : 0.f;
             }
         }
     } else {
@@ -268,7 +277,8 @@ __device__ __forceinline__ void delta_state_io(float (&s)[R], float* column, int
             if constexpr (STORE) {
                 if (ok) column[i0 + e] = s[e];
             } else {
-                s[e] = ok ? column[i0 + e] : 0.f;
+                const float v = column[i0 + e < D ? i0 + e : 0];
+                s[e] = ok ? v : 0.f;
             }
         }
     }
@@ -307,14 +317,20 @@ delta_scan_kernel(const T* __restrict__ packed, long ld, const float* __restrict
         for (int q = 0; q < NVEC; ++q) {
             const int x = tid + q * 256;
             const int tt = x / (5 * DPAD), rem = x % (5 * DPAD), a = rem / DPAD, i = rem % DPAD;
-            gv[q] = (tt < nt && i < D) ? coef[(((size_t)(base + tt) * H + head) * 5 + a) * D + i] : 0.f;
+            // (the load is issued whatever the index, from a clamped address, and its value dropped where
+            // it does not count: loads under a condition would each wait for memory on their own)
+            const bool ok = tt < nt && i < D;
+            const float l = coef[(((size_t)(base + (tt < nt ? tt : 0)) * H + head) * 5 + a) * D + (i < D ? i : 0)];
+            gv[q] = ok ? l : 0.f;
         }
 #pragma unroll
         for (int q = 0; q < NVAL; ++q) {
             const int x = tid + q * 256;
             const int tt = x / COLS, jj = x % COLS;
-            gx[q] = (tt < nt && tt < TT && j0 + jj < D)
-                        ? to_f(packed[(size_t)(base + tt) * ld + 2 * (size_t)inner + (size_t)head * D + j0 + jj]) : 0.f;
+            const bool ok = tt < nt && j0 + jj < D;
+            const float l = to_f(packed[(size_t)(base + (tt < nt ? tt : 0)) * ld + 2 * (size_t)inner + (size_t)head * D
+                                        + (j0 + jj < D ? j0 + jj : 0)]);
+            gx[q] = ok ? l : 0.f;
         }
     };
     auto stash = [&](int buf) {

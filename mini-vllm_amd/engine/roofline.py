@@ -46,6 +46,15 @@ KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
     "mv_attention_decode_fused": (r"\battention_decode(_wave)?_kernel", r"\battention_merge(_range)?_kernel", 2),
     "mv_attention_prefill": (r"\battention_prefill_kernel", None, 1),
     "mv_sample": (r"\bsample(_partial)?_kernel", r"\bsample_kernel", 2),
+    "mv_token_shift": (r"\btoken_shift_kernel", None, 1),
+    "mv_delta_prepare": (r"\bdelta_prepare_kernel", None, 1),
+    "mv_delta_scan": (r"\bdelta_scan_kernel", None, 1),
+    "mv_delta_finish": (r"\bdelta_finish_kernel", None, 1),
+    "mv_delta_step": (r"\bdelta_step_kernel", None, 1),
+    "mv_norm_add_norm": (r"\bnorm_add_norm_kernel", None, 1),
+    "mv_soft_cap": (r"\bsoft_cap_kernel", None, 1),
+    "mv_attention_sigmoid_ref": (r"\battention_sigmoid_kernel", None, 1),
+    "mv_attention_prefill_sigmoid": (r"\battention_prefill_kernel", None, 1),
 }
 _OURS = re.compile("|".join(f"(?:{p})" for spec in KERNELS_OF.values() for p in spec[:2] if p))
 

@@ -212,3 +212,35 @@ def test_greedy_generation(cases, name, dtype):
     # (random weights give flat logits: in bfloat16 most choices are near ties, which only have to lie within the slack)
     assert clear > near if dtype == "float32" else clear >= 20
     llm.manager.check_invariants()
+
+
+def test_command_lines(cases, tmp_path):
+    """``run.py --random-model bolapel-tiny`` prints completions, and ``bin/trace_run`` as a program, fed a
+    trace on its standard input, writes the logits the plain model gives (four state slots by default)."""
+    import ast
+    import json
+    import os
+    import re
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "run.py"), "--random-model", "bolapel-tiny", "--seed", "3",
+                           "--prompt-ids", "5,17,3", "--prompt-ids", "200", "--max-tokens", "5", "--temperature", "0",
+                           "--ignore-eos", "--max-model-len", "64", "--kv-cache-num-blocks", "16",
+                           "--max-num-batched-tokens", "64", "--max-num-batched-seqs", "4"],
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    completions = re.findall(r"Completion:\s*(\[.*?\])", proc.stdout, re.S)
+    assert len(completions) == 2 and all(len(ast.literal_eval(c)) == 5 for c in completions)
+
+    case = cases[("S", "mild")]
+    steps = trace_tools.mixed(case.reqs, prompt_lens_of(case), max_live=4, seed=7)
+    out = tmp_path / "logits"
+    proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", case.dir, "--dtype", "float32", "--out", str(out),
+                           "--max-tokens", str(trace_tools.max_live_tokens(steps))],
+                          input="".join(json.dumps(st) + "\n" for st in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {st['step']}" for st in steps]
+    got = trace_tools.collect(steps, lambda st: (np.fromfile(out / f"{st['step']}.f32", dtype="<f4").reshape(
+        -1, case.cfg["vocab"]) if any(e["want"] for e in st["entries"]) else None))
+    case.check(got, "float32", "S mixed through bin/trace_run")
