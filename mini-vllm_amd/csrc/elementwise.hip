@@ -936,11 +936,11 @@ norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_
         } else {
             const float hf = to_f(hT), prev = to_f(st[c]);
             st[c] = hT;
-            o[c] = from_f<T>(hf + (prev - hf) * mix.at(c));
+            o[c] = from_f<T>(fmaf(prev - hf, mix.at(c), hf));
         }
     };
     if constexpr (NE > 0) {
-        float v[NE], xr[NE], fa[NE], fb[NE], prev[NE];
+        float v[NE], xr[NE], fa[NE], fb[NE], prev[NE], fm[NE];
         float ss = 0.f;
         // every load is issued whatever the column (beyond the row's end the last column is read again and
         // the value dropped): a load under a condition would be a branch with a wait of its own, and the
@@ -954,6 +954,8 @@ norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_
             const int cl = ok ? c : h - 1;
             const float l_prev = to_f(stl[cl]), l_y = to_f(yr[cl]), l_x = x[cl], l_a = wa.at(cl), l_b = wbl.at(cl);
             prev[e] = l_prev;                                          // (st[c] is written by this thread only, below)
+            // (the shift's weight too: a load between the stores at the end would wait for the stores before it)
+            fm[e] = shifted ? mix.at(cl) : 0.f;
             v[e] = ok ? l_y : 0.f;
             xr[e] = l_x;
             fa[e] = l_a + (unit_a ? 1.f : 0.f);
@@ -989,7 +991,7 @@ norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_
                 const T hT = from_f<T>(v[e] * rb * fb[e]);
                 const float hf = to_f(hT);
                 st[c] = hT;
-                o[c] = from_f<T>(hf + (prev[e] - hf) * mix.at(c));
+                o[c] = from_f<T>(fmaf(prev[e] - hf, fm[e], hf));
             }
         }
     } else {
@@ -1023,6 +1025,88 @@ norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_
     }
 }
 
+// The same for rows of a multiple of 8 columns, at most 2048 NC, everything 16-byte aligned: a thread
+// keeps NC chunks of eight neighbouring columns, read and written 16 (bf16) or 32 bytes at a time, all
+// asked for before the first sum (a chunk beyond the row's end reads the row's first again and drops it).
+template <typename T, int NC>
+__global__ void __launch_bounds__(256)
+norm_add_norm_vec_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_a, int unit_a, float* __restrict__ resid,
+                         WeightPtr wb, float eps_b, int unit_b, T* __restrict__ out, int h, ShiftArgs shift) {
+    __shared__ float part_a[4], part_b[4];
+    const int r = blockIdx.x;
+    const int lane = threadIdx.x % MV_WAVE, wave = threadIdx.x / MV_WAVE;
+    const T* yr = y + (size_t)r * ldy;
+    float* x = resid + (size_t)r * h;
+    T* o = out ? out + (size_t)r * h : nullptr;
+    const bool shifted = shift.mix != nullptr && o != nullptr;
+    const int seq = shifted ? shift.token_seq[r] : 0;
+    T* st = (shifted && seq >= 0) ? (T*)shift.state + (size_t)shift.state_slots[seq] * h : nullptr;
+    const WeightPtr mix{shift.mix != nullptr ? shift.mix : wa.p, shift.mix != nullptr ? shift.mix_dtype : wa.dtype};
+    const T* stl = st != nullptr ? st : yr;
+    const WeightPtr wbl = o != nullptr ? wb : wa;
+    float v[NC][8], xr[NC][8], fa[NC][8], fb[NC][8], prev[NC][8], fm[NC][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int d = (threadIdx.x + 256 * c) * 8;
+        const bool ok = d < h;
+        const int dl = ok ? d : 0;
+        Vec8<T>::load(yr + dl, v[c]);
+        Vec8<float>::load(x + dl, xr[c]);
+        wa.at8(dl, fa[c]);
+        wbl.at8(dl, fb[c]);
+        Vec8<T>::load(stl + dl, prev[c]);
+        mix.at8(dl, fm[c]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (!ok) v[c][e] = 0.f;
+            ss = fmaf(v[c][e], v[c][e], ss);
+        }
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) part_a[wave] = ss;
+    __syncthreads();
+    const float ra = 1.f / sqrtf((part_a[0] + part_a[1] + part_a[2] + part_a[3]) / (float)h + eps_a);
+    float ss2 = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int d = (threadIdx.x + 256 * c) * 8;
+        if (d < h) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                v[c][e] = xr[c][e] + v[c][e] * ra * (fa[c][e] + (unit_a ? 1.f : 0.f));
+                ss2 = fmaf(v[c][e], v[c][e], ss2);
+            }
+            Vec8<float>::store(x + d, v[c]);
+        }
+    }
+    if (o == nullptr) return;
+    ss2 = wave_sum(ss2);
+    if (lane == 0) part_b[wave] = ss2;
+    __syncthreads();
+    const float rb = 1.f / sqrtf((part_b[0] + part_b[1] + part_b[2] + part_b[3]) / (float)h + eps_b);
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int d = (threadIdx.x + 256 * c) * 8;
+        if (d >= h) continue;
+        float hn[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) hn[e] = to_f(from_f<T>(v[c][e] * rb * (fb[c][e] + (unit_b ? 1.f : 0.f))));   // as stored
+        if (!shifted) {
+            Vec8<T>::store(o + d, hn);
+        } else if (st == nullptr) {
+            const float zero[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            Vec8<T>::store(o + d, zero);
+        } else {
+            float mixed[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) mixed[e] = fmaf(prev[c][e] - hn[e], fm[c][e], hn[e]);
+            Vec8<T>::store(st + d, hn);
+            Vec8<T>::store(o + d, mixed);
+        }
+    }
+}
+
 extern "C" int mv_norm_add_norm(const void* y, long ldy, const void* wa, int wa_dtype, float eps_a, int unit_a,
                                 float* resid, const void* wb, int wb_dtype, float eps_b, int unit_b, void* out, int n,
                                 int h, const void* shift_mix, int shift_mix_dtype, void* shift_state,
@@ -1039,6 +1123,27 @@ extern "C" int mv_norm_add_norm(const void* y, long ldy, const void* wa, int wa_
     MV_DISPATCH_T(dtype, "norm_add_norm",                                                                            \
                   hipLaunchKernelGGL((norm_add_norm_kernel<T, NE>), dim3(n), dim3(256), 0, stream, (const T*)y, ldy, pa, \
                                      eps_a, unit_a, resid, pb, eps_b, unit_b, (T*)out, h, shift))
+    const size_t esz = mv_dtype_size(dtype), wsz_a = mv_dtype_size(wa_dtype), wsz_b = out ? mv_dtype_size(wb_dtype) : 4,
+                 msz = shift_mix ? mv_dtype_size(shift_mix_dtype) : 4;
+    const bool vec = h % 8 == 0 && h <= 8192 && (ldy * esz) % 16 == 0 && ((uintptr_t)y % 16) == 0 &&
+                     ((uintptr_t)resid % 32) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)wa % (8 * wsz_a)) == 0 &&
+                     ((uintptr_t)wb % (8 * wsz_b)) == 0 && ((uintptr_t)shift_state % 16) == 0 &&
+                     ((uintptr_t)shift_mix % (8 * msz)) == 0;
+    if (vec) {
+#define NAV_LAUNCH(NC)                                                                                                  \
+    MV_DISPATCH_T(dtype, "norm_add_norm",                                                                               \
+                  hipLaunchKernelGGL((norm_add_norm_vec_kernel<T, NC>), dim3(n), dim3(256), 0, stream, (const T*)y, ldy,  \
+                                     pa, eps_a, unit_a, resid, pb, eps_b, unit_b, (T*)out, h, shift))
+        if (h <= 2048) {
+            NAV_LAUNCH(1);
+        } else if (h <= 4096) {
+            NAV_LAUNCH(2);
+        } else {
+            NAV_LAUNCH(4);
+        }
+#undef NAV_LAUNCH
+        return mv_check_launch("norm_add_norm");
+    }
     if (h <= 1024) {
         NAN_LAUNCH(4);
     } else if (h <= 4096) {

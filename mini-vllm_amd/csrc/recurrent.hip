@@ -36,7 +36,7 @@ token_shift_kernel(const T* __restrict__ h, long ldh, T* __restrict__ out, long 
         const T* prev = cur - ldh;
         for (int c = threadIdx.x; c < width; c += blockDim.x) {
             const float x = to_f(cur[c]);
-            o[c] = from_f<T>(x + (to_f(prev[c]) - x) * mix.at(c));
+            o[c] = from_f<T>(fmaf(to_f(prev[c]) - x, mix.at(c), x));
         }
         return;
     }
@@ -46,7 +46,7 @@ token_shift_kernel(const T* __restrict__ h, long ldh, T* __restrict__ out, long 
         const float x = to_f(cur[c]);
         const float p = to_f(st[c]);
         st[c] = tail[c];
-        o[c] = from_f<T>(x + (p - x) * mix.at(c));
+        o[c] = from_f<T>(fmaf(p - x, mix.at(c), x));
     }
 }
 
@@ -498,17 +498,23 @@ delta_step_kernel(const T* __restrict__ packed, long ld, int H, int D, int rank,
     __syncthreads();
     const int sub = tid % L, col = tid / L;
     float* S0 = state + ((size_t)state_slots[seq] * H + head) * (size_t)D * D;
+    // the next columns' state is asked for before this run of columns is stored: a load behind a store
+    // would wait for the store to be acknowledged
+    float s[R], s_next[R];
+    delta_state_io<R, false>(s, S0 + (size_t)(col < D ? col : 0) * D, sub, D, col < D);
     for (int j0 = 0; j0 < D; j0 += COLS) {
         const int j = j0 + col;
         const bool live = j < D;
         float* S = S0 + (size_t)(live ? j : 0) * D;
-        float s[R];
-        delta_state_io<R, false>(s, S, sub, D, live);
+        const int jn = j + COLS;
+        if (j0 + COLS < D) delta_state_io<R, false>(s_next, S0 + (size_t)(jn < D ? jn : 0) * D, sub, D, jn < D);
         DeltaTokenRegs<R> tk;
         delta_read_token<R, DPAD>(tk, &vec[0][0], vals, sub, live ? j : 0);
         const float o = delta_update<R, L>(s, tk);
         delta_state_io<R, true>(s, S, sub, D, live);
         if (live && sub == 0) outs[j] = o;
+#pragma unroll
+        for (int e = 0; e < R; ++e) s[e] = s_next[e];
     }
     __syncthreads();
     // the head's root mean square (a wave over the head, lane by lane, as the finish kernel sums), weight, gate

@@ -51,7 +51,7 @@ KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
     "mv_delta_scan": (r"\bdelta_scan_kernel", None, 1),
     "mv_delta_finish": (r"\bdelta_finish_kernel", None, 1),
     "mv_delta_step": (r"\bdelta_step_kernel", None, 1),
-    "mv_norm_add_norm": (r"\bnorm_add_norm_kernel", None, 1),
+    "mv_norm_add_norm": (r"\bnorm_add_norm(_vec)?_kernel", None, 1),
     "mv_soft_cap": (r"\bsoft_cap_kernel", None, 1),
     "mv_attention_sigmoid_ref": (r"\battention_sigmoid_kernel", None, 1),
     "mv_attention_prefill_sigmoid": (r"\battention_prefill_kernel", None, 1),
