@@ -614,6 +614,20 @@ class Ops:
         self.lib.call("mv_soft_cap", logits.data_ptr(), logits.stride(0) if rows > 1 else cols, rows, cols, float(cap),
                       self._stream())
 
+    @staticmethod
+    def _chunk_priced(plan, chunk: int):
+        """For the ledger: with chunks a request's queries read at most the keys of the chunks they stand in,
+        not its whole context; the plan's key and pair counts are capped accordingly (an upper bound still)."""
+        if plan is None or chunk <= 0:
+            return plan
+        import copy
+        seqs = max(1, len(plan.q_lens) if plan.q_lens else plan.n_seqs)
+        tokens = sum(plan.q_lens) if plan.q_lens else seqs
+        priced = copy.copy(plan)
+        priced.kv_tokens = min(plan.kv_tokens, seqs * chunk + tokens)
+        priced.attention_pairs = min(plan.attention_pairs, tokens * chunk)
+        return priced
+
     def attention_sigmoid(self, q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                           block_table: torch.Tensor, page_size: int, positions: torch.Tensor, token_seq: torch.Tensor,
                           num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float,
@@ -664,14 +678,16 @@ class Ops:
                 and qs % 8 == 0 and os_ % 4 == 0 and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0):
             nt, kw, n_units, n_busy = self._prefill_variant(plan, group, num_kv_heads)
             if nt:
-                self._note_attention("mv_attention_prefill_sigmoid", plan, n, num_heads, num_kv_heads, head_dim, 2)
+                self._note_attention("mv_attention_prefill_sigmoid", self._chunk_priced(plan, c), n, num_heads, num_kv_heads,
+                                     head_dim, 2)
                 self.lib.call("mv_attention_prefill_sigmoid", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                               v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                               positions.data_ptr(), plan.cu_seqlens.data_ptr(), plan.n_seqs, n_units, n_busy, nt, kw,
                               num_heads, num_kv_heads, head_dim, float(scale), w, c, _ptr(bias), _ptr(gate), gate_stride,
                               self._stream())
                 return
-        self._note_attention("mv_attention_sigmoid_ref", plan, n, num_heads, num_kv_heads, head_dim, q.element_size())
+        self._note_attention("mv_attention_sigmoid_ref", self._chunk_priced(plan, c), n, num_heads, num_kv_heads, head_dim,
+                             q.element_size())
         self.lib.call("mv_attention_sigmoid_ref", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size, positions.data_ptr(),
                       token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim, value_dim, float(scale), c, w,
