@@ -45,8 +45,15 @@ BOLA_R = {"architecture": "Bolapel", "vocab": 512, "width": 256, "norm": {"eps":
 # S: no mask (all keys), no rotation, values as large as keys, every head its own keys
 BOLA_S = {"architecture": "Bolapel", "vocab": 150, "width": 48, "norm": {"eps": 2e-5}, "logit_softcap": 5.0,
           "layers": [_attn(2, 2, 24, 24, None, 0, 0.0, 0.2, 64), _delta(2, 12, None)]}
-BOLA = {"P": BOLA_P, "Q": BOLA_Q, "R": BOLA_R, "S": BOLA_S}
-RANKS = {"P": 6, "Q": 5, "R": 32, "S": 3}
+# T: delta-rule layers only (no cache group at all), a head size that is no multiple of four, rank 1
+BOLA_T = {"architecture": "Bolapel", "vocab": 97, "width": 40, "norm": {"eps": 1e-5},
+          "layers": [_delta(2, 30, 56), _delta(3, 16, None)]}
+# U: attention layers only, two readers of one owner, chunks of one token and of three
+BOLA_U = {"architecture": "Bolapel", "vocab": 120, "width": 56, "norm": {"eps": 1e-6}, "logit_softcap": 8.0,
+          "layers": [_attn(2, 1, 16, 8, 5, 8, 300.0, 0.3, 48), _attn(2, 1, 16, 8, 1, 8, 300.0, 0.5, None, kv_from=0),
+                     _attn(2, 1, 16, 8, 3, 8, 300.0, 0.2, 48, kv_from=0)]}
+BOLA = {"P": BOLA_P, "Q": BOLA_Q, "R": BOLA_R, "S": BOLA_S, "T": BOLA_T, "U": BOLA_U}
+RANKS = {"P": 6, "Q": 5, "R": 32, "S": 3, "T": 1, "U": 2}
 
 
 def tensor_shapes(cfg: Dict, rank: int) -> Dict[str, tuple]:

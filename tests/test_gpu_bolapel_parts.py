@@ -119,7 +119,7 @@ def run_delta(ops, packed, t, H, D, rank, eps, state, q_lens, slots, pad_rows=0,
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H, D, rank", [(2, 16, 6), (3, 24, 5), (1, 40, 3), (4, 64, 32), (2, 128, 16), (1, 200, 4),
-                                        (5, 8, 1)])
+                                        (5, 8, 1), (2, 30, 7)])
 def test_delta_rule_mixed_step(dtype, H, D, rank):
     """Requests of 37, 1, 18 and 2 rows in one step, each on a state that earlier tokens left, in slots
     out of order; padding rows and a padding sequence behind them."""
@@ -144,7 +144,7 @@ def test_delta_rule_mixed_step(dtype, H, D, rank):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H, D, rank", [(2, 16, 6), (3, 24, 5), (1, 40, 3), (4, 64, 32), (2, 128, 16), (1, 200, 4),
-                                        (5, 8, 1)])
+                                        (5, 8, 1), (2, 30, 7)])
 def test_delta_rule_step_of_single_tokens(dtype, H, D, rank):
     """Five requests with one token each (slots out of order, a padding row between them): the one fused
     kernel against the plain recurrence, and against the three kernels it stands for."""
