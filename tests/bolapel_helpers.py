@@ -52,8 +52,12 @@ BOLA_T = {"architecture": "Bolapel", "vocab": 97, "width": 40, "norm": {"eps": 1
 BOLA_U = {"architecture": "Bolapel", "vocab": 120, "width": 56, "norm": {"eps": 1e-6}, "logit_softcap": 8.0,
           "layers": [_attn(2, 1, 16, 8, 5, 8, 300.0, 0.3, 48), _attn(2, 1, 16, 8, 1, 8, 300.0, 0.5, None, kv_from=0),
                      _attn(2, 1, 16, 8, 3, 8, 300.0, 0.2, 48, kv_from=0)]}
-BOLA = {"P": BOLA_P, "Q": BOLA_Q, "R": BOLA_R, "S": BOLA_S, "T": BOLA_T, "U": BOLA_U}
-RANKS = {"P": 6, "Q": 5, "R": 32, "S": 3, "T": 1, "U": 2}
+# V: nothing is a multiple of eight (width 50, vocabulary 77, heads of 6 and 10, values of 6, feed-forward 70)
+BOLA_V = {"architecture": "Bolapel", "vocab": 77, "width": 50, "norm": {"eps": 1e-5}, "logit_softcap": 9.0,
+          "layers": [_delta(3, 6, 70), _attn(3, 1, 10, 6, 11, 4, 1000.0, 0.3, 70), _delta(1, 10, None),
+                     _attn(3, 1, 10, 6, 4, 4, 1000.0, 0.4, 70, kv_from=1)]}
+BOLA = {"P": BOLA_P, "Q": BOLA_Q, "R": BOLA_R, "S": BOLA_S, "T": BOLA_T, "U": BOLA_U, "V": BOLA_V}
+RANKS = {"P": 6, "Q": 5, "R": 32, "S": 3, "T": 1, "U": 2, "V": 3}
 
 
 def tensor_shapes(cfg: Dict, rank: int) -> Dict[str, tuple]:

@@ -13,11 +13,11 @@ from helpers import TOL_F32, bf16_tolerance, rel_err, write_model_dir
 
 pytestmark = pytest.mark.gpu
 
-NAMES = ["P", "Q", "R", "S", "T", "U"]
+NAMES = ["P", "Q", "R", "S", "T", "U", "V"]
 # longer than two chunks of every layer, so that chunk edges pass inside prompts and among decoded tokens
 LENGTHS = {"P": [70, 5, 45, 21, 33, 2], "Q": [118, 40, 66, 3, 58], "R": [150, 17, 260, 49], "S": [50, 36, 77, 1],
-           "T": [40, 3, 65], "U": [33, 70, 4]}
-PAGE = {"P": 16, "Q": 8, "R": 16, "S": 16, "T": 16, "U": 8}
+           "T": [40, 3, 65], "U": [33, 70, 4], "V": [44, 9, 61]}
+PAGE = {"P": 16, "Q": 8, "R": 16, "S": 16, "T": 16, "U": 8, "V": 16}
 GAINS = {"sharp": 2.0, "mild": 1.0}
 
 
