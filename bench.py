@@ -32,6 +32,11 @@ default, with prompt lengths uniform in 128..2048 and ``--gen-len`` generated to
 submitted at once under a budget of ``--token-budget`` tokens a step) and prints its own line:
 generated tokens per second over the whole run, with the time of the run and the number of steps.
 
+``--design bolapel`` measures the same things, with the same definitions and the same line, for a Bolapel model
+of the named shape's sizes (``minivllm_amd.config.shapes.bolapel_shape``: the shape's width, feed-forward,
+vocabulary, head counts and number of layers; three delta-rule layers to one attention layer in chunks of
+``--chunk`` tokens), so that the two designs can be read side by side; the default design and workload are Qwen3's.
+
 Weights are seeded random tensors of the named shape and prompts are seeded uniform token ids
 (there is no network for checkpoints or datasets). The reference publishes no number for this
 metric, so ``vs_baseline`` is null.
