@@ -18,6 +18,33 @@
 
 __device__ __forceinline__ float as_sigmoid(float z) { return 1.f / (1.f + expf(-z)); }
 
+// q . k over D channels with the key row read 16 bytes at a time (the caller vouches for D % 8 == 0 and a
+// 16-byte aligned row); the additions run in the order of the channels, as the one-by-one loop's do
+__device__ __forceinline__ float as_dot8(const float* qs, const bf16* krow, int D) {
+    float dot = 0.f;
+    for (int d = 0; d < D; d += 8) {
+        const uint4 u = *reinterpret_cast<const uint4*>(krow + d);
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            dot = fmaf(qs[d + 2 * e], __uint_as_float(w[e] << 16), dot);
+            dot = fmaf(qs[d + 2 * e + 1], __uint_as_float(w[e] & 0xffff0000u), dot);
+        }
+    }
+    return dot;
+}
+__device__ __forceinline__ float as_dot8(const float* qs, const float* krow, int D) {
+    float dot = 0.f;
+    for (int d = 0; d < D; d += 4) {
+        const float4 k = *reinterpret_cast<const float4*>(krow + d);
+        dot = fmaf(qs[d], k.x, dot);
+        dot = fmaf(qs[d + 1], k.y, dot);
+        dot = fmaf(qs[d + 2], k.z, dot);
+        dot = fmaf(qs[d + 3], k.w, dot);
+    }
+    return dot;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(AS_THREADS)
 attention_sigmoid_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out, long out_stride,
@@ -47,6 +74,7 @@ attention_sigmoid_kernel(const T* __restrict__ q, long q_stride, T* __restrict__
     const int hi = pos;
     const int* bt = block_table + (size_t)seq * bt_width;
     const float b = bias ? bias[head] : 0.f;
+    const bool wide_keys = D % 8 == 0 && ((uintptr_t)k_pages % 16) == 0;      // key rows start at multiples of 16 bytes
 
     const T* qrow = q + (size_t)tok * q_stride + (size_t)head * D;
     for (int d = tid; d < D; d += AS_THREADS) qs[d] = to_f(qrow[d]);
@@ -65,7 +93,11 @@ attention_sigmoid_kernel(const T* __restrict__ q, long q_stride, T* __restrict__
             const int slot = j % page_size;
             const T* krow = k_pages + (((size_t)page * Hkv + kvh) * page_size + slot) * D;
             float dot = 0.f;
-            for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f(krow[d]), dot);
+            if (wide_keys) {
+                dot = as_dot8(qs, krow, D);
+            } else {
+                for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f(krow[d]), dot);
+            }
             p = as_sigmoid(dot * scale + b);
             vo = (long)(((size_t)page * Hkv + kvh) * Dv) * page_size + slot;
         }

@@ -99,8 +99,12 @@ def bolapel_tensor_name(config: BolapelConfig, loc: TensorLocation) -> str:
 
 
 def bolapel_ignorable(config: BolapelConfig) -> FrozenSet[str]:
-    # a layer without a feed-forward may still store the two norms around it
-    return frozenset(f"l{i}.{n}" for i, l in enumerate(config.layers) if l.ff is None for n in ("norm2", "norm2b"))
+    # a layer without a feed-forward may still store the two norms around it, and a layer that reads
+    # another layer's keys and values may still store projections of its own: neither is used
+    names = {f"l{i}.{n}" for i, l in enumerate(config.layers) if l.ff is None for n in ("norm2", "norm2b")}
+    names |= {f"l{i}.mix.{n}" for i, l in enumerate(config.layers) if l.type == "attention" and l.kv_from is not None
+              for n in ("k", "v", "k.norm")}
+    return frozenset(names)
 
 
 def bolapel_complete(config: BolapelConfig, source) -> BolapelConfig:
