@@ -227,7 +227,8 @@ def paged(k, v, page_size, n_pages, seed):
     return kp.to(DEV), vp.to(DEV), [int(i) for i in ids]
 
 
-def run_attention(ops, q, k, v, positions, scale, chunk, window, bias, gate, page_size=4, seed=0, with_plan=False):
+def run_attention(ops, q, k, v, positions, scale, chunk, window, bias, gate, page_size=4, seed=0, with_plan=False,
+                  variant=None):
     """``with_plan``: the step is described to the kernels' front end as the engine does (one request of
     these rows, in row 1 of the block table), which lets it pick the MFMA kernel where the sizes allow."""
     from minivllm_amd.engine.step import AttentionPlan
@@ -235,7 +236,7 @@ def run_attention(ops, q, k, v, positions, scale, chunk, window, bias, gate, pag
     plan = None
     if with_plan:
         plan = AttentionPlan(decode_only=n_q == 1, max_q_len=n_q, max_context_len=max(positions) + 1, n_seqs=2,
-                             q_lens=[0, n_q], cu_seqlens=i32([0, 0, n_q]))
+                             q_lens=[0, n_q], cu_seqlens=i32([0, 0, n_q]), prefill_variant=variant)
     Dv = v.shape[2]
     kp, vp, ids = paged(k, v, page_size, 2 * (-(-k.shape[0] // page_size)) + 3, seed)
     table = torch.full((2, len(ids) + 2), -1, dtype=torch.int32)
@@ -321,6 +322,53 @@ def test_mfma_sigmoid_attention_sees_exactly_its_keys(D, chunk, window, page):
                 want[j % D] += 0.5 * (1 + j // D)
             for hd in range(4):
                 assert torch.equal(got[at, hd], want), f"query {i} head {hd} (keys {lo}..{i})"
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("variant", [(1, 1), (2, 1), (1, 2), (2, 2)])
+@pytest.mark.parametrize("chunk, window", [(512, None), (None, None), (300, 77)])
+def test_mfma_sigmoid_attention_long_contexts_every_variant(D, variant, chunk, window):
+    """1,100 tokens, so that a workgroup walks dozens of key blocks, with both column widths and with one
+    and two key groups per workgroup (the two groups' sums are added at the end): rows that name their keys."""
+    dtype = torch.bfloat16
+    ops = ops_for(dtype)
+    n = 1100
+    q = torch.zeros(n, 4, D, dtype=dtype)
+    k = torch.randn(n, 2, D).to(dtype)
+    v = torch.zeros(n, 2, D)
+    for j in range(n):
+        v[j, :, j % D] = 1 + j // D
+    rows = list(range(700, n))
+    got = run_attention(ops, q[rows], k, v.to(dtype), rows, 1.0, chunk, window, torch.zeros(4), None, page_size=16,
+                        with_plan=True, variant=variant).float().cpu()
+    for at, i in enumerate(rows):
+        lo = max(0 if chunk is None else i // chunk * chunk, 0 if window is None else i - window)
+        want = torch.zeros(D)
+        for j in range(lo, i + 1):
+            want[j % D] += 0.5 * (1 + j // D)
+        for hd in range(4):
+            assert torch.equal(got[at, hd], want), f"query {i} head {hd} (keys {lo}..{i})"
+    # random queries, keys, bias and gates over the same context, against the plain function
+    g = torch.Generator().manual_seed(D)
+    q = torch.randn(n, 4, D, generator=g).to(dtype)
+    v = torch.randn(n, 2, D, generator=g).to(dtype)
+    bias = torch.randn(4, generator=g) - 4.0
+    gate = torch.randn(n, 4, generator=g).to(dtype)
+    scale = 1.5 / math.sqrt(D)
+    idx = torch.arange(n)
+    want = plain.chunked_sigmoid_attention(q.double(), k.double(), v.double(), scale, bias.double(), chunk)
+    if window is not None:                                   # the plain function has no window: apply it by hand
+        seen = (idx[None, :] <= idx[:, None]) & (idx[None, :] >= idx[:, None] - window)
+        if chunk is not None:
+            seen &= (idx[None, :] // chunk) == (idx[:, None] // chunk)
+        want = torch.empty(n, 4, D, dtype=torch.float64)
+        for hd in range(4):
+            wgt = torch.sigmoid((q[:, hd].double() @ k[:, hd // 2].double().T) * scale + bias[hd].double()) * seen
+            want[:, hd] = wgt @ v[:, hd // 2].double()
+    want = want * torch.sigmoid(gate.double())[:, :, None]
+    got = run_attention(ops, q[rows], k, v, rows, scale, chunk, window, bias, gate[rows], page_size=16, with_plan=True,
+                        variant=variant)
+    close(got, want[rows], 1e-2, "random rows")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

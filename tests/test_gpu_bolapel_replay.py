@@ -245,3 +245,25 @@ def test_command_lines(cases, tmp_path):
     got = trace_tools.collect(steps, lambda st: (np.fromfile(out / f"{st['step']}.f32", dtype="<f4").reshape(
         -1, case.cfg["vocab"]) if any(e["want"] for e in st["entries"]) else None))
     case.check(got, "float32", "S mixed through bin/trace_run")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_request_past_a_thousand_tokens(cases, dtype):
+    """1,100 tokens through the sizes the MFMA kernels serve: the graphs' context cap doubles at 1,024, the
+    prompt attention walks its keys with two key groups per workgroup, the delta rule's state has run over a
+    thousand tokens; whole, and the last 40 tokens one by one behind a prompt fed in two portions."""
+    case = cases[("R", "mild")]
+    toks = random_tokens(case.cfg, 1100, seed=77)
+    want = plain_logits(case.cfg, case.weights, toks)
+    rows = [0, 1, 47, 48, 511, 512, 1023, 1024, 1059, 1060, 1099]
+    tol = TOL_F32 if dtype == "float32" else bf16_tolerance(
+        max(rel_err(plain_logits_bf16(case.cfg, case.weights, toks)[p], want[p]) for p in rows))
+    steps = [{"step": 0, "entries": [{"id": "w", "tokens": toks, "want": rows}], "end": ["w"]},
+             {"step": 1, "entries": [{"id": "d", "tokens": toks[:1000], "want": [999]}], "end": []},
+             {"step": 2, "entries": [{"id": "d", "tokens": toks[1000:1060], "want": [59]}], "end": []}]
+    steps += [{"step": 3 + i, "entries": [{"id": "d", "tokens": [toks[1060 + i]], "want": [0]}],
+               "end": ["d"] if i == 39 else []} for i in range(40)]
+    got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
+    worst = max(rel_err(row, want[pos]) for (_, pos), row in got.items())
+    print(f"1,100 tokens [{dtype}]: {len(got)} rows, worst relative error {worst:.3e} (allowed {tol:.3e})")
+    assert len(got) == len(rows) + 2 + 40 and worst <= tol
