@@ -479,3 +479,226 @@ class BolapelConfig(ModelConfig):
         if self.max_position_embeddings != (1 << 24):
             d["max_position_embeddings"] = self.max_position_embeddings
         return d
+
+
+# ---------------------------------------------------------------------------------------
+# Dutilix
+# ---------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class DutilixMixer:
+    """The mixer of one Dutilix layer. ``type`` selects which fields count:
+
+    delta             heads, kv_heads (query/key groups), dim (query/key size), vdim, conv (taps)
+    mlstm             heads, dim, vdim, gate_cap
+    latent_attention  heads, dim (unrotated query/key size), rot_dim, vdim, q_rank, kv_rank, scale, rot_base
+    """
+    type: str
+    heads: int
+    dim: int
+    vdim: int
+    kv_heads: int = 0
+    conv: int = 1
+    gate_cap: float = 0.0
+    rot_dim: int = 0
+    rot_base: float = 10000.0
+    q_rank: int = 0
+    kv_rank: int = 0
+    scale: float = 1.0
+
+    def to_dict(self) -> Dict[str, Any]:
+        if self.type == "delta":
+            return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "conv": self.conv}
+        if self.type == "mlstm":
+            return {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "gate_cap": self.gate_cap}
+        return {"heads": self.heads, "dim": self.dim, "rot_dim": self.rot_dim, "vdim": self.vdim, "q_rank": self.q_rank,
+                "kv_rank": self.kv_rank, "scale": self.scale, "rot": {"dims": self.rot_dim, "base": self.rot_base}}
+
+
+@dataclass(frozen=True)
+class DutilixFeedForward:
+    """``kind`` "dense": a gated pair of width ``ff``. "moe": ``experts`` gated pairs of width ``ff`` and ``identity``
+    identity experts behind them, ``top`` used per token, chosen within ``groups_keep`` of ``groups`` groups."""
+    kind: str
+    ff: int
+    experts: int = 0
+    identity: int = 0
+    top: int = 0
+    groups: int = 1
+    groups_keep: int = 1
+
+    def to_dict(self) -> Dict[str, Any]:
+        if self.kind == "dense":
+            return {"kind": "dense", "ff": self.ff}
+        return {"kind": "moe", "expert": {"ff": self.ff},
+                "router": {"experts": self.experts, "identity": self.identity, "top": self.top,
+                           "groups": {"count": self.groups, "keep": self.groups_keep}}}
+
+
+@dataclass(frozen=True)
+class DutilixLayer:
+    mixer: DutilixMixer
+    mlp: Optional[DutilixFeedForward] = None
+
+
+@dataclass(frozen=True)
+class DutilixConfig(ModelConfig):
+    """Dutilix: a pre-norm decoder whose ``layers`` are listed one by one; each has a mixer (``type``:
+    a gated delta rule, an mLSTM matrix memory, or softmax attention over a cached latent) and a
+    feed-forward (dense, a mixture of experts, or none). Keys: ``vocab``, ``width``, ``layers``,
+    ``norm.eps``, ``logit_scale``; the architecture is named by ``architecture``."""
+
+    architecture: ClassVar[str] = "Dutilix"
+
+    vocab_size: int = 0
+    hidden_size: int = 0
+    layers: Tuple[DutilixLayer, ...] = ()
+    norm_eps: float = 1e-6
+    logit_scale: float = 1.0
+    max_position_embeddings: int = 1 << 24
+    dtype: str = "bfloat16"
+    eos_token_ids: Tuple[int, ...] = ()
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any], where: str = "config.json") -> "DutilixConfig":
+        raw_layers = d.get("layers")
+        if not isinstance(raw_layers, (list, tuple)) or not raw_layers:
+            raise ConfigError(f"{where}: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(raw_layers):
+            lw = f"{where}: layers[{i}]"
+            if not isinstance(entry, dict):
+                raise ConfigError(f"{lw} must be an object")
+            kind = entry.get("type")
+            m = _section(entry, "mixer", lw)
+            mw = lw + ".mixer"
+            heads = _require(m, "heads", int, mw)
+            dim = _require(m, "dim", int, mw)
+            vdim = _require(m, "vdim", int, mw)
+            if kind == "delta":
+                kv_heads = m.get("kv_heads")
+                conv = m.get("conv")
+                mixer = DutilixMixer(type=kind, heads=heads, dim=dim, vdim=vdim,
+                                     kv_heads=heads if kv_heads is None else _typed(kv_heads, "kv_heads", int, mw),
+                                     conv=1 if conv is None else _typed(conv, "conv", int, mw))
+            elif kind == "mlstm":
+                mixer = DutilixMixer(type=kind, heads=heads, dim=dim, vdim=vdim,
+                                     gate_cap=_require(m, "gate_cap", float, mw))
+            elif kind == "latent_attention":
+                rot = _section(m, "rot", mw, optional=True)
+                rot_dim = _typed(m.get("rot_dim", 0) or 0, "rot_dim", int, mw)
+                if rot is not None and _require(rot, "dims", int, mw + ".rot") != rot_dim:
+                    raise ConfigError(f"{mw}: rot.dims {rot.get('dims')} differs from rot_dim {rot_dim}; the rotated part "
+                                      f"is rotated as a whole")
+                if rot is None and rot_dim:
+                    raise ConfigError(f"{mw}: rot_dim {rot_dim} without a 'rot' section")
+                mixer = DutilixMixer(type=kind, heads=heads, dim=dim, vdim=vdim, rot_dim=rot_dim,
+                                     rot_base=10000.0 if rot is None else _require(rot, "base", float, mw + ".rot"),
+                                     q_rank=_require(m, "q_rank", int, mw), kv_rank=_require(m, "kv_rank", int, mw),
+                                     scale=_require(m, "scale", float, mw))
+            else:
+                raise ConfigError(f"{lw}: layer type {kind!r} is not supported (delta, mlstm, latent_attention)")
+            mlp = _section(entry, "mlp", lw, optional=True)
+            ff = None
+            if mlp is not None:
+                pw = lw + ".mlp"
+                mk = mlp.get("kind", "dense")
+                if mk == "dense":
+                    ff = DutilixFeedForward(kind="dense", ff=_require(mlp, "ff", int, pw))
+                elif mk == "moe":
+                    expert = _section(mlp, "expert", pw)
+                    router = _section(mlp, "router", pw)
+                    groups = _section(router, "groups", pw + ".router", optional=True)
+                    identity = router.get("identity")
+                    ff = DutilixFeedForward(
+                        kind="moe", ff=_require(expert, "ff", int, pw + ".expert"),
+                        experts=_require(router, "experts", int, pw + ".router"),
+                        identity=0 if identity is None else _typed(identity, "identity", int, pw + ".router"),
+                        top=_require(router, "top", int, pw + ".router"),
+                        groups=1 if groups is None else _require(groups, "count", int, pw + ".router.groups"),
+                        groups_keep=1 if groups is None else _require(groups, "keep", int, pw + ".router.groups"))
+                else:
+                    raise ConfigError(f"{pw}: kind {mk!r} is not supported (dense, moe)")
+            layers.append(DutilixLayer(mixer=mixer, mlp=ff))
+        norm = _section(d, "norm", where)
+        scale = d.get("logit_scale")
+        dtype = d.get("dtype", d.get("torch_dtype", "bfloat16")) or "bfloat16"
+        if str(dtype) not in _DTYPE_NAMES:
+            raise ConfigError(f"{where}: unknown dtype {dtype!r}")
+        eos = d.get("eos_token_id")
+        eos_ids: Tuple[int, ...] = ()
+        if isinstance(eos, int) and not isinstance(eos, bool):
+            eos_ids = (eos,)
+        elif isinstance(eos, (list, tuple)) and all(isinstance(e, int) for e in eos):
+            eos_ids = tuple(eos)
+        elif eos is not None:
+            raise ConfigError(f"{where}: eos_token_id must be an integer or a list of integers, got {eos!r}")
+        max_pos = d.get("max_position_embeddings")
+        cfg = cls(
+            vocab_size=_require(d, "vocab", int, where),
+            hidden_size=_require(d, "width", int, where),
+            layers=tuple(layers),
+            norm_eps=_require(norm, "eps", float, where + ".norm"),
+            logit_scale=1.0 if scale is None else _typed(scale, "logit_scale", float, where),
+            max_position_embeddings=(1 << 24) if max_pos is None else _typed(max_pos, "max_position_embeddings", int, where),
+            dtype=_DTYPE_NAMES[str(dtype)],
+            eos_token_ids=eos_ids,
+        )
+        cfg.validate(where)
+        return cfg
+
+    def validate(self, where: str = "config") -> None:
+        if self.vocab_size <= 0 or self.hidden_size <= 0:
+            raise ConfigError(f"{where}: vocab and width must be positive")
+        if self.norm_eps <= 0:
+            raise ConfigError(f"{where}: norm.eps must be positive, got {self.norm_eps}")
+        for i, l in enumerate(self.layers):
+            lw = f"{where}: layers[{i}]"
+            m = l.mixer
+            if m.heads <= 0 or m.dim <= 0 or m.vdim <= 0:
+                raise ConfigError(f"{lw}: heads, dim and vdim must be positive")
+            if m.type == "delta":
+                if m.kv_heads <= 0 or m.heads % m.kv_heads:
+                    raise ConfigError(f"{lw}: {m.heads} heads are not a multiple of {m.kv_heads} kv_heads")
+                if m.conv < 1:
+                    raise ConfigError(f"{lw}: conv must be >= 1, got {m.conv}")
+            elif m.type == "mlstm":
+                if not m.gate_cap > 0:
+                    raise ConfigError(f"{lw}: gate_cap must be positive, got {m.gate_cap}")
+            else:
+                if m.q_rank <= 0 or m.kv_rank <= 0:
+                    raise ConfigError(f"{lw}: q_rank and kv_rank must be positive")
+                if m.rot_dim < 0 or m.rot_dim % 2:
+                    raise ConfigError(f"{lw}: rot_dim {m.rot_dim} must be even and >= 0")
+                if m.rot_dim and m.rot_base <= 0:
+                    raise ConfigError(f"{lw}: rot.base must be positive")
+            f = l.mlp
+            if f is None:
+                continue
+            if f.ff <= 0:
+                raise ConfigError(f"{lw}: the feed-forward width must be positive")
+            if f.kind == "moe":
+                total = f.experts + f.identity
+                if f.experts < 0 or f.identity < 0 or total < 1:
+                    raise ConfigError(f"{lw}: a router needs at least one expert")
+                if f.groups < 1 or total % f.groups or not (1 <= f.groups_keep <= f.groups):
+                    raise ConfigError(f"{lw}: {total} router outputs do not form {f.groups} equal groups of which "
+                                      f"{f.groups_keep} are kept")
+                if not (1 <= f.top <= total // f.groups * f.groups_keep):
+                    raise ConfigError(f"{lw}: top {f.top} exceeds the experts that can be chosen")
+
+    def to_dict(self) -> Dict[str, Any]:
+        d: Dict[str, Any] = {
+            "architecture": self.architecture,
+            "layers": [{"type": l.mixer.type, "mixer": l.mixer.to_dict(), "mlp": None if l.mlp is None else l.mlp.to_dict()}
+                       for l in self.layers],
+            "norm": {"eps": self.norm_eps},
+            "logit_scale": self.logit_scale,
+            "vocab": self.vocab_size,
+            "width": self.hidden_size,
+            "torch_dtype": self.dtype,
+        }
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids) if len(self.eos_token_ids) > 1 else self.eos_token_ids[0]
+        if self.max_position_embeddings != (1 << 24):
+            d["max_position_embeddings"] = self.max_position_embeddings
+        return d

@@ -637,3 +637,386 @@ extern "C" int mv_delta_finish(const float* raw, const void* packed, long ld, co
                                      (const T*)packed, ld, w, H, D, eps, (T*)out, ldo, n));
     return mv_check_launch("delta_finish");
 }
+
+// =======================================================================================
+// Mixers with a decayed matrix state per head and scalar gates: S is [key size DK][columns DV],
+//     S <- a S;  u = b (v - [READ] S^T k);  S <- S + k u^T;  o = S^T q
+// READ = true is the gated delta rule (a the decay, b the writing strength); READ = false, with a
+// column of ones appended to the values, is the matrix memory of the mLSTM (a, b its stabilised
+// forget and input gates, the extra column its normaliser). The per-token vectors come as floats:
+//     qk    [n][G][2][DK]   query and key of each of the G key groups (head h reads group h / (H / G))
+//     vals  [n][H][DV]      value columns
+//     gates [n][H][4]       a, b, and two numbers the finishing kernel may use
+// and the state as [slots][H][DV][DK], a head's matrix column by column. Prepare kernels make them
+// from the packed projection rows, the scan runs the recurrence request by request, the finish
+// kernel divides each head's output by its root mean square, applies weight and gate.
+// =======================================================================================
+#define MS_MAX_TAPS 16
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+// log(sigmoid(z)) without overflow
+__device__ __forceinline__ float logsigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+// One input of the causal convolution: row r of the step when the request's rows reach back that far,
+// else the request's kept inputs (hist[slot][taps-1][C], the last one the newest).
+template <typename T>
+__device__ __forceinline__ float conv_input(const T* __restrict__ rows, long ld, const T* __restrict__ hist, int C, int taps,
+                                            int first, int r, int c) {
+    if (r >= first) return to_f(rows[(size_t)r * ld + c]);
+    return to_f(hist[(size_t)(taps - 1 + (r - first)) * C + c]);
+}
+
+// ---------------------------------------------------------------------------------------
+// Gated delta rule, prepare. Packed rows: [q (G*DK) | k (G*DK) | v (H*DV) | g (H*DV) | b (H) | a (H)].
+// q, k and v pass a causal convolution over time per channel (taps[c][j], the last tap the current
+// token's) and SiLU; q and k become unit vectors per group (q also times DK^-1/2);
+// b = sigmoid(b), a = exp(-exp(A_log[h]) * softplus(a + dt_bias[h])). Workgroup (row, unit): units
+// 0..G-1 make a group's q and k, units G..G+H-1 a head's values and gates.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(128)
+gdelta_prepare_kernel(const T* __restrict__ packed, long ld, int H, int G, int DK, int DV, int taps, WeightPtr conv_w,
+                      const T* __restrict__ conv_state, WeightPtr a_log, WeightPtr dt_bias, float unit_eps,
+                      const int* __restrict__ token_seq, const int* __restrict__ cu_seqlens,
+                      const int* __restrict__ state_slots, float* __restrict__ qk, float* __restrict__ vals,
+                      float* __restrict__ gates) {
+    __shared__ float scratch[17];
+    const int t = blockIdx.x, unit = blockIdx.y, tid = threadIdx.x;
+    const int seq = token_seq[t];
+    if (seq < 0) return;                                   // a padding row: nobody reads its vectors
+    const int C = 2 * G * DK + H * DV;
+    const int first = cu_seqlens[seq];
+    const T* hist = conv_state + (size_t)state_slots[seq] * (taps - 1) * C;
+    auto conv = [&](int c) {
+        float acc = 0.f;
+        for (int j = 0; j < taps; ++j)
+            acc = fmaf(conv_w.at((size_t)c * taps + j), conv_input(packed, ld, hist, C, taps, first, t - (taps - 1) + j, c), acc);
+        return silu_f(acc);
+    };
+    if (unit < G) {
+        for (int which = 0; which < 2; ++which) {
+            const int c0 = which * G * DK + unit * DK;
+            float* o = qk + (((size_t)t * G + unit) * 2 + which) * DK;
+            float ss = 0.f;
+            for (int d = tid; d < DK; d += 128) {
+                const float x = conv(c0 + d);
+                o[d] = x;                                  // (the thread that wrote it scales it below)
+                ss = fmaf(x, x, ss);
+            }
+            ss = block_sum(ss, scratch);
+            const float inv = (which == 0 ? 1.f / sqrtf((float)DK) : 1.f) / sqrtf(ss + unit_eps);
+            for (int d = tid; d < DK; d += 128) o[d] *= inv;
+        }
+        return;
+    }
+    const int head = unit - G;
+    const int c0 = 2 * G * DK + head * DV;
+    float* o = vals + ((size_t)t * H + head) * DV;
+    for (int d = tid; d < DV; d += 128) o[d] = conv(c0 + d);
+    if (tid == 0) {
+        const T* p = packed + (size_t)t * ld + 2 * (size_t)G * DK + 2 * (size_t)H * DV;
+        float* g = gates + ((size_t)t * H + head) * 4;
+        g[0] = expf(-expf(a_log.at(head)) * softplus_f(to_f(p[H + head]) + dt_bias.at(head)));
+        g[1] = sigmoid_f(to_f(p[head]));
+        g[2] = 0.f;
+        g[3] = 0.f;
+    }
+}
+
+// The convolution's kept inputs after the step: the last taps-1 inputs of each request, from the step's
+// rows and, where the step brought fewer, from what was kept before. Thread (request, channel) reads all
+// it needs before it writes, and no other thread touches its channel.
+template <typename T>
+__global__ void __launch_bounds__(256)
+conv_state_kernel(const T* __restrict__ packed, long ld, int C, int taps, T* __restrict__ conv_state,
+                  const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots) {
+    const int seq = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    const int first = cu_seqlens[seq], end = cu_seqlens[seq + 1];
+    if (end <= first || c >= C) return;
+    T* hist = conv_state + (size_t)state_slots[seq] * (taps - 1) * C;
+    T keep[MS_MAX_TAPS];
+    for (int i = 0; i < taps - 1; ++i) {
+        const int r = end - (taps - 1) + i;
+        keep[i] = r >= first ? packed[(size_t)r * ld + c] : hist[(size_t)(taps - 1 + (r - first)) * C + c];
+    }
+    for (int i = 0; i < taps - 1; ++i) hist[(size_t)i * C + c] = keep[i];
+}
+
+extern "C" int mv_gdelta_prepare(const void* packed, long ld, int n, int n_seqs, int H, int G, int DK, int DV, int taps,
+                                 const void* conv_w, const void* a_log, const void* dt_bias, int weight_dtype,
+                                 void* conv_state, float unit_eps, const int* token_seq, const int* cu_seqlens,
+                                 const int* state_slots, float* qk, float* vals, float* gates, int dtype,
+                                 hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && n_seqs >= 0 && H > 0 && G > 0 && H % G == 0 && DK > 0 && DV > 0,
+               "gdelta_prepare: bad sizes n=%d H=%d G=%d DK=%d DV=%d", n, H, G, DK, DV);
+    MV_REQUIRE(taps >= 1 && taps <= MS_MAX_TAPS, "gdelta_prepare: %d taps, 1 to %d are served", taps, MS_MAX_TAPS);
+    const long C = 2L * G * DK + (long)H * DV;
+    MV_REQUIRE(ld >= C + (long)H * DV + 2L * H, "gdelta_prepare: rows of %ld columns are too short", ld);
+    MV_REQUIRE(mv_valid_dtype(weight_dtype) && packed && conv_w && a_log && dt_bias && (conv_state || taps == 1) && token_seq
+               && cu_seqlens && state_slots && qk && vals && gates, "gdelta_prepare: missing operand");
+    MV_REQUIRE(unit_eps > 0.f && G + H <= 65535 && (C + 255) / 256 <= 65535, "gdelta_prepare: bad constants");
+    if (n == 0) return 0;
+    WeightPtr cw{conv_w, weight_dtype}, al{a_log, weight_dtype}, db{dt_bias, weight_dtype};
+    MV_DISPATCH_T(dtype, "gdelta_prepare",
+                  hipLaunchKernelGGL(gdelta_prepare_kernel<T>, dim3(n, G + H), dim3(128), 0, stream, (const T*)packed, ld, H,
+                                     G, DK, DV, taps, cw, (const T*)conv_state, al, db, unit_eps, token_seq, cu_seqlens,
+                                     state_slots, qk, vals, gates));
+    if (mv_check_launch("gdelta_prepare")) return 1;
+    if (taps > 1 && n_seqs > 0) {
+        MV_DISPATCH_T(dtype, "conv_state",
+                      hipLaunchKernelGGL(conv_state_kernel<T>, dim3(n_seqs, (unsigned)((C + 255) / 256)), dim3(256), 0, stream,
+                                         (const T*)packed, ld, (int)C, taps, (T*)conv_state, cu_seqlens, state_slots));
+        return mv_check_launch("conv_state");
+    }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// mLSTM, gates. Packed rows: [q (H*DK) | k (H*DK) | v (H*DV) | g (H*DV) | i (H) | f (H)]. With the log
+// input gate i = cap tanh((i + i_bias) / cap), the log forget gate f = logsigmoid(cap tanh((f + f_bias) / cap))
+// and the running maximum m (kept per request and head, 0 at the start):
+//     m' = max(f + m, i);   a = exp(f + m - m');   b = exp(i - m');   gates = (a, b, exp(-m'), 0)
+// One wave per (request, head) walks the request's rows 64 at a time: m' is a scan with the
+// associative step (F, I) after (F0, I0) = (F0 + F, max(I0 + F, I)), m' = max(F + m, I).
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(64)
+mlstm_gates_kernel(const T* __restrict__ packed, long ld, int H, long gate_off, WeightPtr i_bias, WeightPtr f_bias, float cap,
+                   float* __restrict__ max_state, const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots,
+                   float* __restrict__ gates) {
+    const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const int first = cu_seqlens[seq], end = cu_seqlens[seq + 1];
+    if (end <= first) return;
+    float* ms = max_state + (size_t)state_slots[seq] * H + head;
+    float m = *ms;
+    const float bi = i_bias.at(head), bf = f_bias.at(head);
+    for (int base = first; base < end; base += 64) {
+        const int t = base + lane;
+        const bool live = t < end;
+        const T* p = packed + (size_t)(live ? t : first) * ld + gate_off;
+        const float gi = cap * tanhf((to_f(p[head]) + bi) / cap);
+        const float gf = logsigmoid_f(cap * tanhf((to_f(p[H + head]) + bf) / cap));
+        float F = live ? gf : 0.f, I = live ? gi : -INFINITY;         // rows past the end change nothing
+        for (int o = 1; o < 64; o <<= 1) {
+            const float Fp = __shfl_up(F, o, 64), Ip = __shfl_up(I, o, 64);
+            if (lane >= o) {
+                I = fmaxf(Ip + F, I);
+                F = Fp + F;
+            }
+        }
+        const float m_new = fmaxf(F + m, I);
+        float m_prev = __shfl_up(m_new, 1, 64);
+        if (lane == 0) m_prev = m;
+        if (live) {
+            float* g = gates + ((size_t)t * H + head) * 4;
+            g[0] = expf(gf + m_prev - m_new);
+            g[1] = expf(gi - m_new);
+            g[2] = expf(-m_new);
+            g[3] = 0.f;
+        }
+        m = __shfl(m_new, 63, 64);
+    }
+    if (lane == 0) *ms = m;
+}
+
+// mLSTM, the vectors of the scan: q * DK^-1/2 and k as floats, the values with a one behind them.
+template <typename T>
+__global__ void __launch_bounds__(128)
+mlstm_prepare_kernel(const T* __restrict__ packed, long ld, int H, int DK, int DV, const int* __restrict__ token_seq,
+                     float* __restrict__ qk, float* __restrict__ vals) {
+    const int t = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+    if (token_seq[t] < 0) return;
+    const T* p = packed + (size_t)t * ld;
+    float* o = qk + ((size_t)t * H + head) * 2 * DK;
+    const float qs = 1.f / sqrtf((float)DK);
+    for (int d = tid; d < DK; d += 128) {
+        o[d] = to_f(p[(size_t)head * DK + d]) * qs;
+        o[DK + d] = to_f(p[(size_t)(H + head) * DK + d]);
+    }
+    float* v = vals + ((size_t)t * H + head) * (DV + 1);
+    for (int d = tid; d < DV; d += 128) v[d] = to_f(p[2 * (size_t)H * DK + (size_t)head * DV + d]);
+    if (tid == 0) v[DV] = 1.f;
+}
+
+extern "C" int mv_mlstm_prepare(const void* packed, long ld, int n, int n_seqs, int H, int DK, int DV, const void* i_bias,
+                                const void* f_bias, int weight_dtype, float cap, float* max_state, const int* token_seq,
+                                const int* cu_seqlens, const int* state_slots, float* qk, float* vals, float* gates,
+                                int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && n_seqs >= 0 && H > 0 && DK > 0 && DV > 0, "mlstm_prepare: bad sizes n=%d H=%d DK=%d DV=%d", n, H, DK, DV);
+    const long gate_off = 2L * H * DK + 2L * H * DV;
+    MV_REQUIRE(ld >= gate_off + 2L * H, "mlstm_prepare: rows of %ld columns are too short", ld);
+    MV_REQUIRE(mv_valid_dtype(weight_dtype) && packed && i_bias && f_bias && max_state && token_seq && cu_seqlens && state_slots
+               && qk && vals && gates, "mlstm_prepare: missing operand");
+    MV_REQUIRE(cap > 0.f && H <= 65535, "mlstm_prepare: bad constants");
+    if (n == 0 || n_seqs == 0) return 0;
+    WeightPtr ib{i_bias, weight_dtype}, fb{f_bias, weight_dtype};
+    MV_DISPATCH_T(dtype, "mlstm_gates",
+                  hipLaunchKernelGGL(mlstm_gates_kernel<T>, dim3(n_seqs, H), dim3(64), 0, stream, (const T*)packed, ld, H,
+                                     gate_off, ib, fb, cap, max_state, cu_seqlens, state_slots, gates));
+    if (mv_check_launch("mlstm_gates")) return 1;
+    MV_DISPATCH_T(dtype, "mlstm_prepare",
+                  hipLaunchKernelGGL(mlstm_prepare_kernel<T>, dim3(n, H), dim3(128), 0, stream, (const T*)packed, ld, H, DK, DV,
+                                     token_seq, qk, vals));
+    return mv_check_launch("mlstm_prepare");
+}
+
+// ---------------------------------------------------------------------------------------
+// The scan. A workgroup of 256 threads owns 256 / L columns of one head of one request, L
+// neighbouring lanes share a column and keep R of its DK rows each (as in the delta rule's scan
+// above). The vectors of a run of tokens are staged in LDS; the additions of a token depend on
+// nothing but the sizes, so a token computed alone has the bits it has inside a prompt.
+// ---------------------------------------------------------------------------------------
+template <int R, int L, bool READ>
+__global__ void __launch_bounds__(256)
+state_scan_kernel(const float* __restrict__ qk, const float* __restrict__ vals, const float* __restrict__ gates,
+                  float* __restrict__ state, const int* __restrict__ cu_seqlens, const int* __restrict__ state_slots, int H,
+                  int G, int DK, int DV, float* __restrict__ out) {
+    constexpr int DPAD = L * R;
+    constexpr int COLS = 256 / L;
+    constexpr int TT = DPAD > 128 ? 4 : (DPAD > 64 ? 8 : 16);
+    __shared__ __attribute__((aligned(16))) float sv[TT][2][DPAD];
+    __shared__ float sx[TT][COLS];
+    __shared__ float sg[TT][2];
+    const int seq = blockIdx.x, head = blockIdx.y, j0 = blockIdx.z * COLS;
+    const int begin = cu_seqlens[seq], end = cu_seqlens[seq + 1];
+    if (end <= begin) return;
+    const int tid = threadIdx.x, sub = tid % L, col = tid / L;
+    const int j = j0 + col;
+    const bool live = j < DV;
+    const int group = head / (H / G);
+    float* S = state + (((size_t)state_slots[seq] * H + head) * DV + (live ? j : 0)) * (size_t)DK;
+    float s[R];
+    delta_state_io<R, false>(s, S, sub, DK, live);
+    for (int base = begin; base < end; base += TT) {
+        const int nt = min(TT, end - base);
+        __syncthreads();                                   // the run before has been read
+        for (int x = tid; x < nt * 2 * DPAD; x += 256) {
+            const int tt = x / (2 * DPAD), rem = x % (2 * DPAD), a = rem / DPAD, i = rem % DPAD;
+            sv[tt][a][i] = i < DK ? qk[(((size_t)(base + tt) * G + group) * 2 + a) * DK + i] : 0.f;
+        }
+        for (int x = tid; x < nt * COLS; x += 256) {
+            const int tt = x / COLS, jj = x % COLS;
+            sx[tt][jj] = j0 + jj < DV ? vals[((size_t)(base + tt) * H + head) * DV + j0 + jj] : 0.f;
+        }
+        if (tid < nt * 2) sg[tid / 2][tid % 2] = gates[((size_t)(base + tid / 2) * H + head) * 4 + tid % 2];
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float a = sg[tt][0], b = sg[tt][1], v = sx[tt][col];
+            float q[R], k[R];
+#pragma unroll
+            for (int e = 0; e < R; ++e) {
+                q[e] = sv[tt][0][sub * R + e];
+                k[e] = sv[tt][1][sub * R + e];
+            }
+            float u = v;
+            if constexpr (READ) {
+                float read = 0.f;
+#pragma unroll
+                for (int e = 0; e < R; ++e) read = fmaf(k[e], s[e], read);
+                u = v - a * lanes_sum<L>(read);
+            }
+            u *= b;
+            float o = 0.f;
+#pragma unroll
+            for (int e = 0; e < R; ++e) {
+                s[e] = fmaf(a, s[e], k[e] * u);
+                o = fmaf(q[e], s[e], o);
+            }
+            o = lanes_sum<L>(o);
+            if (live && sub == 0) out[((size_t)(base + tt) * H + head) * DV + j] = o;
+        }
+    }
+    delta_state_io<R, true>(s, S, sub, DK, live);
+}
+
+extern "C" int mv_state_scan(const float* qk, const float* vals, const float* gates, float* state, const int* cu_seqlens,
+                             const int* state_slots, int n_seqs, int n, int H, int G, int DK, int DV, int read,
+                             float* out, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && n_seqs >= 0 && H > 0 && G > 0 && H % G == 0 && DK > 0 && DV > 0,
+               "state_scan: bad sizes n=%d seqs=%d H=%d G=%d DK=%d DV=%d", n, n_seqs, H, G, DK, DV);
+    MV_REQUIRE(DK <= 256, "state_scan: key size %d exceeds the supported maximum 256", DK);
+    MV_REQUIRE(qk && vals && gates && state && cu_seqlens && state_slots && out, "state_scan: missing operand");
+    int R = 0, L = 0;
+    delta_scan_shape(DK, R, L);
+    const int cols = 256 / L;
+    MV_REQUIRE(H <= 65535 && (DV + cols - 1) / cols <= 65535, "state_scan: too many heads or columns");
+    if (n == 0 || n_seqs == 0) return 0;
+    dim3 grid(n_seqs, H, (DV + cols - 1) / cols);
+#define MS_LAUNCH(RR, LL)                                                                                                  \
+    if (read)                                                                                                              \
+        hipLaunchKernelGGL((state_scan_kernel<RR, LL, true>), grid, dim3(256), 0, stream, qk, vals, gates, state, cu_seqlens, \
+                           state_slots, H, G, DK, DV, out);                                                                \
+    else                                                                                                                   \
+        hipLaunchKernelGGL((state_scan_kernel<RR, LL, false>), grid, dim3(256), 0, stream, qk, vals, gates, state,         \
+                           cu_seqlens, state_slots, H, G, DK, DV, out);
+    if (R == 4 && L == 4) {
+        MS_LAUNCH(4, 4)
+    } else if (R == 4 && L == 8) {
+        MS_LAUNCH(4, 8)
+    } else if (R == 4 && L == 16) {
+        MS_LAUNCH(4, 16)
+    } else if (R == 8 && L == 16) {
+        MS_LAUNCH(8, 16)
+    } else {
+        MS_LAUNCH(16, 16)
+    }
+#undef MS_LAUNCH
+    return mv_check_launch("state_scan");
+}
+
+// ---------------------------------------------------------------------------------------
+// Finish. One wave per (row, head): the head's DV outputs (of DVS columns the scan wrote), with
+// `normaliser` divided by max(|column DV|, gates[2]) + denom_eps first; then
+//     y[d] = o[d] / sqrt(mean(o^2) + eps) * weight[shared ? d : head * DV + d] * act(g[head * DV + d])
+// act = SiLU (silu_gate) or the logistic function; g at column g_off of the packed rows.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+state_finish_kernel(const float* __restrict__ raw, const float* __restrict__ gates, const T* __restrict__ packed, long ld,
+                    long g_off, WeightPtr weight, int shared_weight, int silu_gate, int normaliser, float denom_eps, int H,
+                    int DV, int DVS, float eps, const int* __restrict__ token_seq, T* __restrict__ out, long ldo, int n) {
+    const int lane = threadIdx.x % MV_WAVE;
+    const long unit = (long)blockIdx.x * 4 + threadIdx.x / MV_WAVE;
+    if (unit >= (long)n * H) return;
+    const int t = (int)(unit / H), head = (int)(unit % H);
+    T* y = out + (size_t)t * ldo + (size_t)head * DV;
+    if (token_seq[t] < 0) {
+        for (int d = lane; d < DV; d += MV_WAVE) y[d] = from_f<T>(0.f);
+        return;
+    }
+    const float* o = raw + ((size_t)t * H + head) * DVS;
+    float scale = 1.f;
+    if (normaliser) scale = 1.f / (fmaxf(fabsf(o[DV]), gates[((size_t)t * H + head) * 4 + 2]) + denom_eps);
+    float ss = 0.f;
+    for (int d = lane; d < DV; d += MV_WAVE) {
+        const float x = o[d] * scale;
+        ss = fmaf(x, x, ss);
+    }
+    ss = wave_sum(ss);
+    const float rinv = scale / sqrtf(ss / (float)DV + eps);
+    const T* g = packed + (size_t)t * ld + g_off + (size_t)head * DV;
+    for (int d = lane; d < DV; d += MV_WAVE) {
+        const float z = to_f(g[d]);
+        const float act = silu_gate ? silu_f(z) : sigmoid_f(z);
+        y[d] = from_f<T>(o[d] * rinv * weight.at(shared_weight ? d : (size_t)head * DV + d) * act);
+    }
+}
+
+extern "C" int mv_state_finish(const float* raw, const float* gates, const void* packed, long ld, long g_off,
+                               const void* weight, int weight_dtype, int shared_weight, int silu_gate, int normaliser,
+                               float denom_eps, int n, int H, int DV, float eps, const int* token_seq, void* out, long ldo,
+                               int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && H > 0 && DV > 0 && eps > 0.f, "state_finish: bad sizes n=%d H=%d DV=%d", n, H, DV);
+    MV_REQUIRE(g_off >= 0 && ld >= g_off + (long)H * DV && ldo >= (long)H * DV, "state_finish: row pitches too small");
+    MV_REQUIRE(mv_valid_dtype(weight_dtype) && raw && gates && packed && weight && token_seq && out, "state_finish: missing operand");
+    if (n == 0) return 0;
+    const long units = (long)n * H;
+    WeightPtr w{weight, weight_dtype};
+    MV_DISPATCH_T(dtype, "state_finish",
+                  hipLaunchKernelGGL(state_finish_kernel<T>, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, stream, raw, gates,
+                                     (const T*)packed, ld, g_off, w, shared_weight, silu_gate, normaliser, denom_eps, H, DV,
+                                     DV + (normaliser ? 1 : 0), eps, token_seq, (T*)out, ldo, n));
+    return mv_check_launch("state_finish");
+}

@@ -144,6 +144,43 @@ _OPTIONAL_SIGNATURES = {
     "mv_attention_prefill_sigmoid": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                              c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                              c_float, c_int, c_int, c_void_p, c_void_p, c_long, c_void_p]),
+    # packed, ld, n, n_seqs, H, G, DK, DV, taps, conv_w, a_log, dt_bias, weight_dtype, conv_state, unit_eps, token_seq,
+    # cu_seqlens, state_slots, qk, vals, gates, dtype, stream
+    "mv_gdelta_prepare": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                                  c_void_p, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_int, c_void_p]),
+    # packed, ld, n, n_seqs, H, DK, DV, i_bias, f_bias, weight_dtype, cap, max_state, token_seq, cu_seqlens, state_slots,
+    # qk, vals, gates, dtype, stream
+    "mv_mlstm_prepare": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float,
+                                 c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    # qk, vals, gates, state, cu_seqlens, state_slots, n_seqs, n, H, G, DK, DV, read, out, stream
+    "mv_state_scan": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                              c_int, c_int, c_void_p, c_void_p]),
+    # raw, gates, packed, ld, g_off, weight, weight_dtype, shared_weight, silu_gate, normaliser, denom_eps, n, H, DV, eps,
+    # token_seq, out, ldo, dtype, stream
+    "mv_state_finish": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_long, c_void_p, c_int, c_int, c_int, c_int, c_float,
+                                c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_long, c_int, c_void_p]),
+    # packed, ld, n, QR, R, DR, wq, wkv, weight_dtype, eps, table, table_rows, positions, token_seq, block_table, bt_width,
+    # page_size, cq, ldq, pages, dtype, stream
+    "mv_latent_prepare": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
+                                  c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_int,
+                                  c_void_p]),
+    # x, ldx, ldx_head, w, weight_dtype, n, H, IN, OUT, y, ldy, ldy_head, tail, table, positions, gate, ldg, token_seq, mode,
+    # dtype, stream
+    "mv_head_linear": (c_int, [c_void_p, c_long, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_long, c_int,
+                               c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p]),
+    # q, ldq, out, ldo, pages, block_table, bt_width, page_size, positions, token_seq, n, H, R, DR, scale, dtype, stream
+    "mv_attention_latent": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p,
+                                    c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
+    # logits, ld, n, E, correction, weight_dtype, groups, keep, top, sum_eps, dense, ids, weights, stream
+    "mv_moe_route": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
+                             c_void_p, c_void_p]),
+    # gate_up, ld, dense, ld_dense, n, E, F, act, dtype, stream
+    "mv_moe_swiglu_scale": (c_int, [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p]),
+    # y, ldy, h, ldh, dense, ld_dense, first, count, n, width, set, dtype, stream
+    "mv_moe_identity_add": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_int, c_void_p]),
+    "mv_scale_f32": (c_int, [c_void_p, c_long, c_int, c_int, c_float, c_void_p]),
     "mv_launch_empty": (c_int, [c_int, c_int, c_void_p, c_void_p]),
 }
 

@@ -559,6 +559,283 @@ class Ops:
                       weight.data_ptr(), _weight_code(weight, "delta norm weight"), n, heads, dim, float(eps),
                       out.data_ptr(), out.stride(0) if n > 1 else inner, self.code, self._stream())
 
+    # ------------------------------------------------------------------------------------
+    # mixers with a decayed matrix state per head and scalar gates (gated delta rule, mLSTM)
+    def _state_vectors(self, n: int, heads: int, groups: int, dk: int, dvs: int, qk: torch.Tensor, vals: torch.Tensor,
+                       gates: torch.Tensor, what: str) -> None:
+        for t, shape, name in ((qk, (n, groups, 2, dk), "queries and keys"), (vals, (n, heads, dvs), "values"),
+                               (gates, (n, heads, 4), "gates")):
+            _dev(t, name)
+            if t.dtype != torch.float32 or tuple(t.shape) != shape or not t.is_contiguous():
+                raise KernelLibraryError(f"{what}: {name} must be contiguous float32 {shape}, got {tuple(t.shape)} {t.dtype}")
+
+    def gated_delta_prepare(self, packed: torch.Tensor, heads: int, groups: int, dk: int, dv: int, taps: int,
+                            conv_w: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                            conv_state: Optional[torch.Tensor], unit_eps: float, token_seq: torch.Tensor,
+                            cu_seqlens: torch.Tensor, state_slots: torch.Tensor, n_seqs: int, qk: torch.Tensor,
+                            vals: torch.Tensor, gates: torch.Tensor) -> None:
+        """From rows [q (groups*dk) | k (groups*dk) | v (heads*dv) | g | b (heads) | a (heads)]: q, k, v through a
+        causal convolution of ``taps`` taps per channel (conv_w [channels, taps], last tap the current token) and
+        SiLU; q and k unit vectors per group (q times dk^-1/2); gates[..., 0] = exp(-exp(a_log) softplus(a + dt_bias)),
+        gates[..., 1] = sigmoid(b). conv_state [slots, taps-1, channels] holds each request's last inputs: read for
+        the rows in front of the step, then advanced."""
+        self._act(packed, "delta rows")
+        n, C = packed.shape[0], 2 * groups * dk + heads * dv
+        if packed.dim() != 2 or packed.stride(1) != 1 or packed.shape[1] < C + heads * dv + 2 * heads:
+            raise KernelLibraryError(f"gated_delta_prepare: rows {tuple(packed.shape)} are too short")
+        self._state_vectors(n, heads, groups, dk, dv, qk, vals, gates, "gated_delta_prepare")
+        for t, shape, name in ((conv_w, (C, taps), "convolution taps"), (a_log, (heads,), "A_log"), (dt_bias, (heads,), "dt_bias")):
+            _dev(t, name)
+            if tuple(t.shape) != shape or not t.is_contiguous() or t.dtype != conv_w.dtype:
+                raise KernelLibraryError(f"gated_delta_prepare: {name} must be a contiguous {shape} tensor of the taps' dtype")
+        if taps > 1:
+            self._act(conv_state, "convolution state")
+            if conv_state.dim() != 3 or tuple(conv_state.shape[1:]) != (taps - 1, C) or not conv_state.is_contiguous():
+                raise KernelLibraryError(f"gated_delta_prepare: the convolution's state must be [slots, {taps - 1}, {C}]")
+        self._ints(n, token_seq=(token_seq, n), cu_seqlens=(cu_seqlens, n_seqs + 1), state_slots=(state_slots, n_seqs))
+        self._note("mv_gdelta_prepare", n * (C + 2 * heads) * packed.element_size() + self._size(qk, vals, gates), 2 * n * C * taps + 8 * n * C)
+        self.lib.call("mv_gdelta_prepare", packed.data_ptr(), packed.stride(0) if n > 1 else packed.shape[1], n, n_seqs, heads,
+                      groups, dk, dv, taps, conv_w.data_ptr(), a_log.data_ptr(), dt_bias.data_ptr(),
+                      _weight_code(conv_w, "convolution taps"), _ptr(conv_state), float(unit_eps), token_seq.data_ptr(),
+                      cu_seqlens.data_ptr(), state_slots.data_ptr(), qk.data_ptr(), vals.data_ptr(), gates.data_ptr(),
+                      self.code, self._stream())
+
+    def mlstm_prepare(self, packed: torch.Tensor, heads: int, dk: int, dv: int, i_bias: torch.Tensor, f_bias: torch.Tensor,
+                      cap: float, max_state: torch.Tensor, token_seq: torch.Tensor, cu_seqlens: torch.Tensor,
+                      state_slots: torch.Tensor, n_seqs: int, qk: torch.Tensor, vals: torch.Tensor, gates: torch.Tensor) -> None:
+        """From rows [q | k (heads*dk each) | v | g (heads*dv each) | i | f (heads each)]: q * dk^-1/2 and k as floats,
+        the values with a one behind them (vals [n, heads, dv + 1]), and the stabilised gates: with
+        i' = cap tanh((i + i_bias)/cap), f' = logsigmoid(cap tanh((f + f_bias)/cap)) and the running maximum
+        m' = max(f' + m, i') (max_state [slots, heads], read and advanced), gates = (exp(f' + m - m'), exp(i' - m'), exp(-m'), 0)."""
+        self._act(packed, "mlstm rows")
+        n = packed.shape[0]
+        if packed.dim() != 2 or packed.stride(1) != 1 or packed.shape[1] < 2 * heads * (dk + dv) + 2 * heads:
+            raise KernelLibraryError(f"mlstm_prepare: rows {tuple(packed.shape)} are too short")
+        self._state_vectors(n, heads, heads, dk, dv + 1, qk, vals, gates, "mlstm_prepare")
+        for t, name in ((i_bias, "input gate bias"), (f_bias, "forget gate bias")):
+            _dev(t, name)
+            if t.numel() != heads or not t.is_contiguous() or t.dtype != i_bias.dtype:
+                raise KernelLibraryError(f"mlstm_prepare: the {name} must hold {heads} numbers")
+        _dev(max_state, "running maximum")
+        if max_state.dtype != torch.float32 or max_state.dim() != 2 or max_state.shape[1] != heads or not max_state.is_contiguous():
+            raise KernelLibraryError(f"mlstm_prepare: the running maximum must be float32 [slots, {heads}]")
+        self._ints(n, token_seq=(token_seq, n), cu_seqlens=(cu_seqlens, n_seqs + 1), state_slots=(state_slots, n_seqs))
+        self._note("mv_mlstm_prepare", n * (2 * heads * dk + heads * dv + 2 * heads) * packed.element_size() + self._size(qk, vals, gates),
+                   40 * n * heads)
+        self.lib.call("mv_mlstm_prepare", packed.data_ptr(), packed.stride(0) if n > 1 else packed.shape[1], n, n_seqs, heads, dk,
+                      dv, i_bias.data_ptr(), f_bias.data_ptr(), _weight_code(i_bias, "gate bias"), float(cap),
+                      max_state.data_ptr(), token_seq.data_ptr(), cu_seqlens.data_ptr(), state_slots.data_ptr(), qk.data_ptr(),
+                      vals.data_ptr(), gates.data_ptr(), self.code, self._stream())
+
+    def state_scan(self, qk: torch.Tensor, vals: torch.Tensor, gates: torch.Tensor, state: torch.Tensor,
+                   cu_seqlens: torch.Tensor, state_slots: torch.Tensor, n_seqs: int, heads: int, groups: int, dk: int,
+                   dvs: int, read: bool, out: torch.Tensor) -> None:
+        """Per request and head, token by token: S <- a S; u = b (v - [read] S^T k); S <- S + k u^T; out = S^T q, with
+        (a, b) = gates[..., :2]. state float32 [slots, heads, dvs, dk] (a head's matrix column by column) is read and
+        left advanced; out float32 [n, heads, dvs]."""
+        n = vals.shape[0]
+        self._state_vectors(n, heads, groups, dk, dvs, qk, vals, gates, "state_scan")
+        _dev(state, "matrix state"); _dev(out, "scan output")
+        if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dvs, dk) or not state.is_contiguous():
+            raise KernelLibraryError(f"state_scan: the state must be float32 [slots, {heads}, {dvs}, {dk}]")
+        if out.dtype != torch.float32 or tuple(out.shape) != (n, heads, dvs) or not out.is_contiguous():
+            raise KernelLibraryError(f"state_scan: the output must be float32 [{n}, {heads}, {dvs}]")
+        self._ints(n, cu_seqlens=(cu_seqlens, n_seqs + 1), state_slots=(state_slots, n_seqs))
+        self._note("mv_state_scan", self._size(qk, vals, gates, out) + 2 * min(n_seqs, max(n, 1)) * heads * dvs * dk * 4,
+                   (6 if read else 4) * n * heads * dvs * dk)
+        self.lib.call("mv_state_scan", qk.data_ptr(), vals.data_ptr(), gates.data_ptr(), state.data_ptr(), cu_seqlens.data_ptr(),
+                      state_slots.data_ptr(), n_seqs, n, heads, groups, dk, dvs, int(bool(read)), out.data_ptr(), self._stream())
+
+    def state_finish(self, raw: torch.Tensor, gates: torch.Tensor, packed: torch.Tensor, gate_offset: int, weight: torch.Tensor,
+                     heads: int, dv: int, eps: float, token_seq: torch.Tensor, out: torch.Tensor, shared_weight: bool,
+                     silu_gate: bool, normaliser: bool = False, denom_eps: float = 0.0) -> None:
+        """out[t, h] = o / rms(o) * weight * act(g) per head, o = raw[t, h, :dv]; with ``normaliser`` o is first divided
+        by max(|raw[t, h, dv]|, gates[t, h, 2]) + denom_eps. ``weight`` holds dv numbers shared by the heads or
+        heads*dv; act is SiLU or the logistic function; g are ``heads*dv`` columns of ``packed`` from ``gate_offset``."""
+        self._act(packed, "mixer rows"); self._act(out, "mixer output"); _dev(weight, "output norm weight")
+        n, dvs = packed.shape[0], dv + (1 if normaliser else 0)
+        if raw.dtype != torch.float32 or tuple(raw.shape) != (n, heads, dvs) or not raw.is_contiguous():
+            raise KernelLibraryError(f"state_finish: the scan's output must be float32 [{n}, {heads}, {dvs}]")
+        if gates.dtype != torch.float32 or tuple(gates.shape) != (n, heads, 4) or not gates.is_contiguous():
+            raise KernelLibraryError("state_finish: gates must be float32 [n, heads, 4]")
+        if tuple(out.shape) != (n, heads * dv) or out.stride(1) != 1 or packed.shape[1] < gate_offset + heads * dv \
+                or weight.numel() != (dv if shared_weight else heads * dv) or not weight.is_contiguous():
+            raise KernelLibraryError("state_finish: operands do not fit")
+        self._ints(n, token_seq=(token_seq, n))
+        self._note("mv_state_finish", self._size(raw, out) + n * heads * dv * packed.element_size(), 8 * n * heads * dv)
+        self.lib.call("mv_state_finish", raw.data_ptr(), gates.data_ptr(), packed.data_ptr(),
+                      packed.stride(0) if n > 1 else packed.shape[1], int(gate_offset), weight.data_ptr(),
+                      _weight_code(weight, "output norm weight"), int(shared_weight), int(silu_gate), int(normaliser),
+                      float(denom_eps), n, heads, dv, float(eps), token_seq.data_ptr(), out.data_ptr(),
+                      out.stride(0) if n > 1 else heads * dv, self.code, self._stream())
+
+    # ------------------------------------------------------------------------------------
+    # attention over a cached latent
+    def latent_prepare(self, packed: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, q_norm: torch.Tensor,
+                       kv_norm: torch.Tensor, eps: float, table: Optional[torch.Tensor], positions: torch.Tensor,
+                       token_seq: torch.Tensor, block_table: torch.Tensor, page_size: int, q_latent: torch.Tensor,
+                       pages: torch.Tensor) -> None:
+        """From rows [dq (q_rank) | dkv (kv_rank + rot_dim) | ...]: q_latent = rmsnorm(dq) * q_norm; the row's cache
+        entry [rmsnorm(dkv[:kv_rank]) * kv_norm | rot(dkv[kv_rank:])] goes to pages [pages, page_size, kv_rank + rot_dim]
+        at the row's position (``table``: float32 [positions, rot_dim] = cat(cos, sin), pairs i, i + rot_dim/2)."""
+        self._act(packed, "latent rows"); self._act(q_latent, "query latent"); self._act(pages, "latent pages")
+        n = packed.shape[0]
+        if packed.dim() != 2 or packed.stride(1) != 1 or packed.shape[1] < q_rank + kv_rank + rot_dim:
+            raise KernelLibraryError(f"latent_prepare: rows {tuple(packed.shape)} are too short")
+        if tuple(q_latent.shape) != (n, q_rank) or q_latent.stride(1) != 1:
+            raise KernelLibraryError(f"latent_prepare: the query latent must be [{n}, {q_rank}]")
+        if pages.dim() != 3 or tuple(pages.shape[1:]) != (page_size, kv_rank + rot_dim) or not pages.is_contiguous():
+            raise KernelLibraryError(f"latent_prepare: pages must be [pages, {page_size}, {kv_rank + rot_dim}]")
+        for t, size, name in ((q_norm, q_rank, "query latent norm"), (kv_norm, kv_rank, "latent norm")):
+            _dev(t, name)
+            if t.numel() != size or not t.is_contiguous() or t.dtype != q_norm.dtype:
+                raise KernelLibraryError(f"latent_prepare: the {name} weight must hold {size} numbers")
+        rows = 0
+        if rot_dim:
+            _dev(table, "rotary table")
+            if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != rot_dim or not table.is_contiguous():
+                raise KernelLibraryError(f"latent_prepare: the rotary table must be float32 [positions, {rot_dim}]")
+            rows = table.shape[0]
+        _dev(block_table, "block table")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+            raise KernelLibraryError("latent_prepare: the block table must be contiguous int32 [sequences, width]")
+        self._ints(n, positions=(positions, n), token_seq=(token_seq, n))
+        self._note("mv_latent_prepare", n * (q_rank + kv_rank + rot_dim) * 2 * packed.element_size(), 8 * n * (q_rank + kv_rank + rot_dim))
+        self.lib.call("mv_latent_prepare", packed.data_ptr(), packed.stride(0) if n > 1 else packed.shape[1], n, q_rank, kv_rank,
+                      rot_dim, q_norm.data_ptr(), kv_norm.data_ptr(), _weight_code(q_norm, "latent norm"), float(eps),
+                      _ptr(table), rows, positions.data_ptr(), token_seq.data_ptr(), block_table.data_ptr(),
+                      block_table.shape[1], page_size, q_latent.data_ptr(), q_latent.stride(0) if n > 1 else q_rank,
+                      pages.data_ptr(), self.code, self._stream())
+
+    def head_linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, token_seq: torch.Tensor, tail: int = 0,
+                    table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
+                    gate: Optional[torch.Tensor] = None) -> None:
+        """Per head h: out[t, h, :OUT] = x[t, h, :IN] @ w[h] with w [heads, IN, OUT]. x [n, heads, IN + tail] in the
+        activation type gives out float32 [n, heads, OUT + tail], the ``tail`` last inputs copied behind the outputs
+        and rotated by the row's position (``table`` as for ``latent_prepare``); x float32 [n, heads, IN] gives out
+        [n, heads * OUT] in the activation type, multiplied by sigmoid(gate [n, heads * OUT]) when a gate is given."""
+        _dev(x, "head_linear input"); _dev(w, "head_linear weight"); _dev(out, "head_linear output")
+        if w.dim() != 3 or not w.is_contiguous() or x.dim() != 3 or x.stride(2) != 1 or x.stride(1) != x.shape[2]:
+            raise KernelLibraryError("head_linear: x [n, heads, width] and a contiguous w [heads, IN, OUT] are needed")
+        n, H = x.shape[0], w.shape[0]
+        IN, OUT = w.shape[1], w.shape[2]
+        self._ints(n, token_seq=(token_seq, n))
+        if out.dim() == 3 and x.dtype == self.dtype and out.dtype == torch.float32 and gate is None:
+            mode = 0
+            if tuple(x.shape) != (n, H, IN + tail) or tuple(out.shape) != (n, H, OUT + tail) or not out.is_contiguous():
+                raise KernelLibraryError(f"head_linear: {tuple(x.shape)} x {tuple(w.shape)} -> {tuple(out.shape)} does not fit")
+            ldy, ldy_head = out.stride(0) if n > 1 else H * (OUT + tail), OUT + tail
+            if tail:
+                _dev(table, "rotary table")
+                if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != tail or not table.is_contiguous():
+                    raise KernelLibraryError(f"head_linear: the rotary table must be float32 [positions, {tail}]")
+                self._ints(n, positions=(positions, n))
+        elif out.dim() == 2 and x.dtype == torch.float32 and out.dtype == self.dtype and tail == 0:
+            mode = 1
+            if tuple(x.shape) != (n, H, IN) or tuple(out.shape) != (n, H * OUT) or out.stride(1) != 1:
+                raise KernelLibraryError(f"head_linear: {tuple(x.shape)} x {tuple(w.shape)} -> {tuple(out.shape)} does not fit")
+            ldy, ldy_head = out.stride(0) if n > 1 else H * OUT, OUT
+            if gate is not None:
+                self._act(gate, "output gate")
+                if tuple(gate.shape) != (n, H * OUT) or gate.stride(1) != 1:
+                    raise KernelLibraryError("head_linear: the gate must be [n, heads * OUT]")
+        else:
+            raise KernelLibraryError(f"head_linear: {x.dtype} -> {out.dtype} with these options is not served")
+        self._note("mv_head_linear", self._size(x, w, out), 2 * n * H * IN * OUT)
+        self.lib.call("mv_head_linear", x.data_ptr(), x.stride(0) if n > 1 else H * x.shape[2], x.shape[2], w.data_ptr(),
+                      _weight_code(w, "head_linear weight"), n, H, IN, OUT, out.data_ptr(), ldy, ldy_head, tail, _ptr(table),
+                      _ptr(positions), _ptr(gate), (gate.stride(0) if n > 1 else H * OUT) if gate is not None else 0,
+                      token_seq.data_ptr(), mode, self.code, self._stream())
+
+    def attention_latent(self, q: torch.Tensor, out: torch.Tensor, pages: torch.Tensor, block_table: torch.Tensor,
+                         page_size: int, positions: torch.Tensor, token_seq: torch.Tensor, heads: int, kv_rank: int,
+                         rot_dim: int, scale: float, plan=None) -> None:
+        """Causal softmax attention of q float32 [n, heads, kv_rank + rot_dim] over the cached rows [latent | rotated
+        key part] of each row's request (pages [pages, page_size, kv_rank + rot_dim]); out float32 [n, heads, kv_rank] is
+        the weighted sum of the latents."""
+        _dev(q, "latent queries"); _dev(out, "latent attention output"); self._act(pages, "latent pages")
+        n, dk = q.shape[0], kv_rank + rot_dim
+        if q.dtype != torch.float32 or tuple(q.shape) != (n, heads, dk) or not q.is_contiguous():
+            raise KernelLibraryError(f"attention_latent: queries must be float32 [{n}, {heads}, {dk}]")
+        if out.dtype != torch.float32 or tuple(out.shape) != (n, heads, kv_rank) or not out.is_contiguous():
+            raise KernelLibraryError(f"attention_latent: the output must be float32 [{n}, {heads}, {kv_rank}]")
+        if pages.dim() != 3 or tuple(pages.shape[1:]) != (page_size, dk) or not pages.is_contiguous():
+            raise KernelLibraryError(f"attention_latent: pages must be [pages, {page_size}, {dk}]")
+        _dev(block_table, "block table")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+            raise KernelLibraryError("attention_latent: the block table must be contiguous int32 [sequences, width]")
+        self._ints(n, positions=(positions, n), token_seq=(token_seq, n))
+        kv_tokens = plan.kv_tokens if plan is not None else 0
+        pairs = plan.attention_pairs if plan is not None else 0
+        self._note("mv_attention_latent", self._size(q, out) + kv_tokens * dk * pages.element_size(),
+                   2 * pairs * heads * (dk + kv_rank))
+        self.lib.call("mv_attention_latent", q.data_ptr(), heads * dk, out.data_ptr(), heads * kv_rank, pages.data_ptr(),
+                      block_table.data_ptr(), block_table.shape[1], page_size, positions.data_ptr(), token_seq.data_ptr(),
+                      n, heads, kv_rank, rot_dim, float(scale), self.code, self._stream())
+
+    # ------------------------------------------------------------------------------------
+    # mixture of experts
+    def moe_route(self, logits: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
+                  sum_eps: float, dense: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> None:
+        """From float32 router logits [n, E]: scores = softmax over E; the ``top`` largest of scores + correction among the
+        experts of the ``keep`` groups (of ``groups`` equal runs of neighbours) whose largest such number is largest are
+        chosen; a chosen expert's weight is its score / (sum of the chosen scores + sum_eps). dense float32 [n, E] gets the
+        weights (zero elsewhere), ids int32 / weights float32 [n, top] the chosen experts in the order of choice."""
+        _dev(logits, "router logits")
+        n, E = logits.shape
+        if logits.dtype != torch.float32 or logits.stride(1) != 1:
+            raise KernelLibraryError("moe_route: float32 logits [n, E] are needed")
+        for t, shape, dt, name in ((dense, (n, E), torch.float32, "dense weights"), (ids, (n, top), torch.int32, "ids"),
+                                   (weights, (n, top), torch.float32, "weights")):
+            _dev(t, name)
+            if t.dtype != dt or tuple(t.shape) != shape or not t.is_contiguous():
+                raise KernelLibraryError(f"moe_route: {name} must be contiguous {dt} {shape}")
+        if correction is not None:
+            _dev(correction, "router correction")
+            if correction.numel() != E or not correction.is_contiguous():
+                raise KernelLibraryError(f"moe_route: the correction must hold {E} numbers")
+        self._note("mv_moe_route", self._size(logits, dense, ids, weights), 20 * n * E)
+        self.lib.call("mv_moe_route", logits.data_ptr(), logits.stride(0) if n > 1 else E, n, E, _ptr(correction),
+                      _weight_code(correction, "router correction") if correction is not None else DTYPE_F32, groups, keep,
+                      top, float(sum_eps), dense.data_ptr(), ids.data_ptr(), weights.data_ptr(), self._stream())
+
+    def moe_swiglu_scale(self, gate_up: torch.Tensor, dense: torch.Tensor, experts: int, ff: int, out: torch.Tensor) -> None:
+        """out[t, e, c] = dense[t, e] * silu(gate_up[t, e*ff + c]) * gate_up[t, experts*ff + e*ff + c] (zero where the
+        weight is zero, whatever the products hold)."""
+        self._act(gate_up, "gate_up"); self._act(out, "expert activations"); _dev(dense, "dense weights")
+        n = gate_up.shape[0]
+        if tuple(gate_up.shape) != (n, 2 * experts * ff) or gate_up.stride(1) != 1 or tuple(out.shape) != (n, experts * ff) \
+                or not out.is_contiguous() or dense.dtype != torch.float32 or dense.shape[0] != n or dense.shape[1] < experts \
+                or dense.stride(1) != 1:
+            raise KernelLibraryError("moe_swiglu_scale: operands do not fit")
+        self._note("mv_moe_swiglu_scale", self._size(gate_up, out), 8 * out.numel())
+        self.lib.call("mv_moe_swiglu_scale", gate_up.data_ptr(), gate_up.stride(0) if n > 1 else 2 * experts * ff, dense.data_ptr(),
+                      dense.stride(0) if n > 1 else dense.shape[1], n, experts, ff, out.data_ptr(), self.code, self._stream())
+
+    def moe_identity_add(self, y: torch.Tensor, h: torch.Tensor, dense: torch.Tensor, first: int, count: int,
+                         overwrite: bool = False) -> None:
+        """y[t] += (dense[t, first:first+count] summed) * h[t]; with ``overwrite`` y is set instead."""
+        self._act(y, "feed-forward output"); self._act(h, "feed-forward input"); _dev(dense, "dense weights")
+        n, width = y.shape
+        if tuple(h.shape) != (n, width) or y.stride(1) != 1 or h.stride(1) != 1 or dense.dtype != torch.float32 \
+                or dense.shape[0] != n or dense.shape[1] < first + count or dense.stride(1) != 1:
+            raise KernelLibraryError("moe_identity_add: operands do not fit")
+        self._note("mv_moe_identity_add", 2 * self._size(y) + self._size(h), 2 * n * width)
+        self.lib.call("mv_moe_identity_add", y.data_ptr(), y.stride(0) if n > 1 else width, h.data_ptr(),
+                      h.stride(0) if n > 1 else width, dense.data_ptr(), dense.stride(0) if n > 1 else dense.shape[1], first,
+                      count, n, width, int(overwrite), self.code, self._stream())
+
+    def scale_f32(self, x: torch.Tensor, factor: float) -> None:
+        """In place on float32 [rows, cols]: x <- x * factor."""
+        _dev(x, "rows")
+        if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
+            raise KernelLibraryError("scale_f32: float32 rows with a contiguous last dimension are needed")
+        rows, cols = x.shape
+        if rows == 0:
+            return
+        self._note("mv_scale_f32", 2 * self._size(x), rows * cols)
+        self.lib.call("mv_scale_f32", x.data_ptr(), x.stride(0) if rows > 1 else cols, rows, cols, float(factor), self._stream())
+
     def norm_add_norm(self, y: torch.Tensor, norm_y, resid: torch.Tensor, norm_next, out: Optional[torch.Tensor],
                       shift: Optional[tuple] = None) -> None:
         """resid += rmsnorm(y) * w (``norm_y`` = (weight, eps, unit_offset)); with ``norm_next`` of the same

@@ -2,4 +2,5 @@ from .registry import (Architecture, config_from_dict, get_architecture, load_co
                        registered_architectures, unregister_architecture)
 from . import qwen3  # registers "Qwen3ForCausalLM"
 from . import bolapel  # registers "Bolapel"
+from . import dutilix  # registers "Dutilix"
 from .causal_lm import CausalLM, expected_tensors

@@ -10,4 +10,7 @@ from .attention import Attention, AttentionSpec
 from .mlp import SwiGLU, SwiGLUSpec
 from .block import PreNormBlock, PreNormBlockSpec, SandwichBlock, SandwichBlockSpec
 from .delta_rule import DeltaRule, DeltaRuleSpec
-from .io import CappedHeadSpec, CappedLinearHead, LinearHead, TokenEmbedding
+from .matrix_state import MLSTM, GatedDelta, GatedDeltaSpec, MLSTMSpec
+from .latent_attention import LatentAttention, LatentAttentionSpec, LatentNeed
+from .moe import RoutedExperts, RoutedExpertsSpec
+from .io import CappedHeadSpec, CappedLinearHead, LinearHead, ScaledHeadSpec, ScaledLinearHead, TokenEmbedding

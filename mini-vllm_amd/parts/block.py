@@ -24,9 +24,15 @@ class PreNormBlock(Block):
     into the next norm's kernel through the stream's pending delta."""
     norm_slots: Tuple[str, ...] = ("mixer", "ffn")
 
+    @classmethod
+    def slots_for(cls, has_ffn: bool) -> Tuple[str, ...]:
+        return cls.norm_slots if has_ffn else cls.norm_slots[:1]
+
     def __init__(self, spec: PreNormBlockSpec, norms: Dict[str, Norm], mixer: Mixer, ffn: FeedForward):
         self.norm_mixer = norms["mixer"]
-        self.norm_ffn = norms["ffn"]
+        self.norm_ffn = norms.get("ffn")
+        if ffn is not None and self.norm_ffn is None:
+            raise ValueError("a pre-norm block with a feed-forward needs the norm in front of it")
         self.mixer = mixer
         self.ffn = ffn
 
@@ -43,6 +49,9 @@ class PreNormBlock(Block):
         # fuse it into that product; a part that ends with one may be offered the add and the norm
         # that follow it, to fold them into that product, when the part behind that norm can go on
         # from rows that are not yet divided by their root mean square
+        if self.ffn is None:             # a layer without a feed-forward: the mixer's half alone
+            self._run(stream, ctx, self.norm_mixer, self.mixer, next_norm, next_part, (call,))
+            return
         self._run(stream, ctx, self.norm_mixer, self.mixer, self.norm_ffn, self.ffn, (call,))
         self._run(stream, ctx, self.norm_ffn, self.ffn, next_norm, next_part, ())
 

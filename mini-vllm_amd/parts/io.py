@@ -77,3 +77,23 @@ class CappedLinearHead(LinearHead):
         logits = super().forward(h, ctx)
         self.rt.ops.soft_cap(logits, self.spec.cap)
         return logits
+
+
+@dataclass(frozen=True)
+class ScaledHeadSpec(PartSpec):
+    """A linear head whose logits are multiplied by a constant."""
+    kind = "scaled_linear_head"
+    vocab_size: int = 0
+    hidden_size: int = 0
+    scale: float = 1.0
+
+
+@register_head(ScaledHeadSpec.kind)
+class ScaledLinearHead(LinearHead):
+    spec_class = ScaledHeadSpec
+
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        logits = super().forward(h, ctx)
+        if self.spec.scale != 1.0:
+            self.rt.ops.scale_f32(logits, self.spec.scale)
+        return logits

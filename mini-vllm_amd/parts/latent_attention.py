@@ -1,0 +1,128 @@
+"""Softmax attention whose keys and values are linear maps of one cached latent per token.
+
+From the mixer's input h:
+
+    c_q = rmsnorm(W_dq h) * w_q_norm,   q = W_uq c_q                  (heads x [plain_dim | rot_dim])
+    W_dkv h = [down (kv_rank) | key part (rot_dim)]
+    c   = rmsnorm(down) * w_kv_norm                                    (the latent)
+    k_rot = rot(key part, position)                                    (one for all heads)
+
+Head h's key is [W_uk,h c | k_rot] and its value W_uv,h c; the score of query i and key j <= i is
+(q_plain . W_uk c_j + rot(q_rot) . k_rot,j) * scale, softmax over the visible keys. The heads'
+outputs are concatenated, multiplied by sigmoid(W_g h) when ``output_gate`` is set, and projected
+by W_o.
+
+Only [c | k_rot] is cached, one row of ``kv_rank + rot_dim`` numbers per token
+(``LatentNeed``). Keys and values are never expanded: the query is carried into the latent's space
+(W_uk,h^T q_plain), attention runs on the cached rows with the latent as the value, and W_uv,h is
+applied to the weighted sum of latents. Norms, rotation, scores, weights and sums are float32.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from .base import CacheNeed, KeepAll, Mixer, PartSpec, Retention, Runtime, TensorDecl, register_mixer
+
+
+@dataclass(frozen=True)
+class LatentNeed(CacheNeed):
+    """One row per token: the latent and the rotated key part side by side."""
+    retention: Retention
+    width: int
+
+    def page_shapes(self, page_size: int) -> Dict[str, Tuple[int, ...]]:
+        return {"latent": (page_size, self.width)}
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec(PartSpec):
+    kind = "latent_attention"
+    hidden_size: int = 0
+    num_heads: int = 0
+    plain_dim: int = 0                  # query/key channels of a head that are not rotated
+    rot_dim: int = 0                    # rotated channels: of each query head, and of the one shared key part
+    value_dim: int = 0
+    q_rank: int = 0
+    kv_rank: int = 0
+    scale: float = 1.0
+    norm_eps: float = 1e-6              # of the two latent norms
+    output_gate: bool = False
+    position: Optional[PartSpec] = None     # a rotary encoding over rot_dim channels (None: rot_dim must be 0)
+
+
+@register_mixer(LatentAttentionSpec.kind)
+class LatentAttention(Mixer):
+    spec_class = LatentAttentionSpec
+
+    @classmethod
+    def tensors(cls, spec: LatentAttentionSpec) -> Dict[str, TensorDecl]:
+        hid, H = spec.hidden_size, spec.num_heads
+        t = {"dq": TensorDecl((spec.q_rank, hid)), "dq_norm": TensorDecl((spec.q_rank,), init="ones_normal"),
+             "uq": TensorDecl((H * (spec.plain_dim + spec.rot_dim), spec.q_rank)),
+             "dkv": TensorDecl((spec.kv_rank + spec.rot_dim, hid)), "dkv_norm": TensorDecl((spec.kv_rank,), init="ones_normal"),
+             "uk": TensorDecl((H * spec.plain_dim, spec.kv_rank)), "uv": TensorDecl((H * spec.value_dim, spec.kv_rank)),
+             "o": TensorDecl((hid, H * spec.value_dim))}
+        if spec.output_gate:
+            t["g"] = TensorDecl((H * spec.value_dim, hid))
+        return t
+
+    @classmethod
+    def cache_need(cls, spec: LatentAttentionSpec) -> Optional[CacheNeed]:
+        return LatentNeed(retention=KeepAll(), width=spec.kv_rank + spec.rot_dim)
+
+    def __init__(self, spec: LatentAttentionSpec, tensors: Dict[str, torch.Tensor], rt: Runtime, position: Optional[object] = None):
+        if min(spec.num_heads, spec.plain_dim, spec.value_dim, spec.q_rank, spec.kv_rank) < 1 or spec.rot_dim < 0 or spec.rot_dim % 2:
+            raise ValueError(f"latent attention: bad sizes {spec}")
+        self.spec, self.rt = spec, rt
+        self.table = None
+        if spec.rot_dim:
+            rotary = position.rotary() if position is not None else None
+            if rotary is None or rotary[1] or rotary[0].shape[1] != spec.rot_dim:
+                raise ValueError("latent attention rotates its rot_dim channels in half-split pairs: it needs a rotary "
+                                 "encoding over exactly rot_dim channels")
+            self.table = rotary[0]
+        names = ["dq", "dkv"] + (["g"] if spec.output_gate else [])
+        dtypes = {tensors[p].dtype for p in names}
+        if len(dtypes) != 1:
+            raise ValueError(f"latent attention: the projections are stored in different dtypes {dtypes}; cannot pack them")
+        blocks = [tensors[p] for p in names]
+        self.gate_offset = spec.q_rank + spec.kv_rank + spec.rot_dim
+        pad = (-sum(b.shape[0] for b in blocks)) % 8
+        if pad:
+            blocks.append(torch.zeros((pad, spec.hidden_size), dtype=blocks[0].dtype, device=blocks[0].device))
+        self.w_packed = torch.cat(blocks, dim=0).contiguous()
+        self.width = self.w_packed.shape[0]
+        self.q_norm = tensors["dq_norm"]
+        self.kv_norm = tensors["dkv_norm"].to(self.q_norm.dtype)
+        self.w_uq = tensors["uq"]
+        # [heads, inputs, outputs]: the stored W_uk is that already; W_uv is stored [heads * value_dim, kv_rank]
+        self.w_uk = tensors["uk"].view(spec.num_heads, spec.plain_dim, spec.kv_rank).contiguous()
+        self.w_uv = tensors["uv"].view(spec.num_heads, spec.value_dim, spec.kv_rank).transpose(1, 2).contiguous()
+        self.w_o = tensors["o"]
+
+    def forward(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
+        spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
+        n, H, R, dr = x.shape[0], spec.num_heads, spec.kv_rank, spec.rot_dim
+        packed = ws.get("latent.packed", (n, self.width), rt.dtype)
+        ops.gemm(x, self.w_packed, packed)
+        kv = ctx.kv(call)
+        pages = kv.pages["latent"]
+        cq = ws.get("latent.cq", (n, spec.q_rank), rt.dtype)
+        ops.latent_prepare(packed, spec.q_rank, R, dr, self.q_norm, self.kv_norm, spec.norm_eps, self.table, ctx.positions,
+                           ctx.token_seq, kv.block_table, kv.page_size, cq, pages)
+        q = ws.get("latent.q", (n, H * (spec.plain_dim + dr)), rt.dtype)
+        ops.gemm(cq, self.w_uq, q)
+        qa = ws.get("latent.qa", (n, H, R + dr), torch.float32)
+        ops.head_linear(q.view(n, H, spec.plain_dim + dr), self.w_uk, qa, ctx.token_seq, tail=dr, table=self.table,
+                        positions=ctx.positions)
+        mixed = ws.get("latent.mixed", (n, H, R), torch.float32)
+        ops.attention_latent(qa, mixed, pages, kv.block_table, kv.page_size, ctx.positions, ctx.token_seq, H, R, dr,
+                             spec.scale, plan=ctx.attention_plan)
+        heads = ws.get("latent.heads", (n, H * spec.value_dim), rt.dtype)
+        gate = packed[:, self.gate_offset:self.gate_offset + H * spec.value_dim] if spec.output_gate else None
+        ops.head_linear(mixed, self.w_uv, heads, ctx.token_seq, gate=gate)
+        y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
+        return ops.gemm(heads, self.w_o, y, defer_sum=True) or y

@@ -1,0 +1,98 @@
+"""A mixture of gated feed-forward experts behind a softmax router.
+
+Router logits z = W_router x in float32; scores s = softmax(z) over all router outputs. The last
+``identity_experts`` outputs are identity experts (their output is x itself, they have no tensors), the
+others are gated SiLU pairs down_e(silu(gate_e x) * (up_e x)). A token uses ``top`` experts: those with
+the largest s + correction (the correction steers the choice only, never the weights), restricted to
+the ``keep_groups`` of ``groups`` equal runs of neighbouring router outputs whose largest such number is
+largest (outputs of other groups cannot be chosen whatever their number). The weights are the chosen
+experts' scores divided by their sum (+ weight_sum_eps); the result is the weighted sum of the
+chosen experts' outputs.
+
+How it runs: gate and up matrices of all experts form one packed product and all down matrices one
+second product; between them one kernel applies SiLU, the up factor and the router's weight (zero
+for experts that were not chosen) before the single rounding, so the second product sums exactly the
+chosen experts. Everything is decided on the device; nothing about a step's routing reaches the host.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict
+
+import torch
+
+from .base import FeedForward, PartSpec, Runtime, TensorDecl, register_feed_forward
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec(PartSpec):
+    kind = "routed_swiglu"
+    hidden_size: int = 0
+    expert_size: int = 0                 # width of one expert's gated pair
+    num_experts: int = 0                 # experts with tensors
+    identity_experts: int = 0            # router outputs behind them whose expert is the identity
+    top: int = 1
+    groups: int = 1
+    keep_groups: int = 1
+    correction: bool = False             # a stored number per router output added to the scores for the choice
+    weight_sum_eps: float = 1e-20
+
+    @property
+    def router_outputs(self) -> int:
+        return self.num_experts + self.identity_experts
+
+
+@register_feed_forward(RoutedExpertsSpec.kind)
+class RoutedExperts(FeedForward):
+    spec_class = RoutedExpertsSpec
+
+    @classmethod
+    def tensors(cls, spec: RoutedExpertsSpec) -> Dict[str, TensorDecl]:
+        t = {"router": TensorDecl((spec.router_outputs, spec.hidden_size))}
+        if spec.correction:
+            t["correction"] = TensorDecl((spec.router_outputs,), init="zeros_normal")
+        for e in range(spec.num_experts):
+            t[f"gate.{e}"] = TensorDecl((spec.expert_size, spec.hidden_size))
+            t[f"up.{e}"] = TensorDecl((spec.expert_size, spec.hidden_size))
+            t[f"down.{e}"] = TensorDecl((spec.hidden_size, spec.expert_size))
+        return t
+
+    def __init__(self, spec: RoutedExpertsSpec, tensors: Dict[str, torch.Tensor], rt: Runtime):
+        E = spec.router_outputs
+        if spec.num_experts < 0 or spec.identity_experts < 0 or E < 1 or spec.groups < 1 or E % spec.groups \
+                or not (1 <= spec.keep_groups <= spec.groups) or not (1 <= spec.top <= E // spec.groups * spec.keep_groups):
+            raise ValueError(f"routed experts: bad sizes {spec}")
+        self.spec, self.rt = spec, rt
+        self.w_router = tensors["router"]
+        self.correction = tensors.get("correction")
+        n_e = spec.num_experts
+        if n_e:
+            dtypes = {tensors[f"{k}.{e}"].dtype for e in range(n_e) for k in ("gate", "up", "down")}
+            if len(dtypes) != 1:
+                raise ValueError(f"routed experts: the experts are stored in different dtypes {dtypes}; cannot pack them")
+            # rows: every expert's gate block, then every expert's up block; the down matrices side by side
+            self.w_gate_up = torch.cat([tensors[f"gate.{e}"] for e in range(n_e)]
+                                       + [tensors[f"up.{e}"] for e in range(n_e)], dim=0).contiguous()
+            self.w_down = torch.cat([tensors[f"down.{e}"] for e in range(n_e)], dim=1).contiguous()
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
+        if not isinstance(x, torch.Tensor):
+            x = x.materialize()
+        n, E, n_e, F = x.shape[0], spec.router_outputs, spec.num_experts, spec.expert_size
+        logits = ws.get("moe.logits", (n, E), torch.float32)
+        ops.gemm(x, self.w_router, logits)
+        dense = ws.get("moe.dense", (n, E), torch.float32)
+        ids = ws.get("moe.ids", (n, spec.top), torch.int32)
+        weights = ws.get("moe.weights", (n, spec.top), torch.float32)
+        ops.moe_route(logits, self.correction, spec.groups, spec.keep_groups, spec.top, spec.weight_sum_eps, dense, ids, weights)
+        y = ws.get("ffn.out", (n, spec.hidden_size), rt.dtype)
+        if n_e:
+            gu = ws.get("moe.gate_up", (n, 2 * n_e * F), rt.dtype)
+            ops.gemm(x, self.w_gate_up, gu)
+            act = ws.get("moe.act", (n, n_e * F), rt.dtype)
+            ops.moe_swiglu_scale(gu, dense, n_e, F, act)
+            ops.gemm(act, self.w_down, y)
+        if spec.identity_experts or not n_e:
+            ops.moe_identity_add(y, x, dense, n_e, spec.identity_experts, overwrite=not n_e)
+        return y
