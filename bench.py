@@ -81,6 +81,9 @@ def build_llm(args, shape, layers, max_seqs=None, token_budget=None, num_pages=N
     if getattr(args, "design", "qwen3") == "bolapel":
         from minivllm_amd.config.shapes import bolapel_shape
         raw = dict(bolapel_shape(args.shape, layers, chunk=args.chunk), torch_dtype=args.dtype)
+    elif getattr(args, "design", "qwen3") == "dutilix":
+        from minivllm_amd.config.shapes import dutilix_shape
+        raw = dict(dutilix_shape(args.shape, layers, experts=args.experts, top=args.top), torch_dtype=args.dtype)
     else:
         raw = dict(shape, architectures=["Qwen3ForCausalLM"], num_hidden_layers=layers,
                    max_position_embeddings=40960, torch_dtype=args.dtype)
@@ -361,13 +364,91 @@ def bench_bolapel(args, llm, cfg, layers, layers_full, item) -> int:
     return 0
 
 
+def dutilix_numbers(llm, cfg, item):
+    """From the loaded model: elements of all tensors; of the matrices every token multiplies with (the experts'
+    counted by the share of them a token uses); of all expert matrices; bytes of state a request reads and
+    writes a step; cache bytes a token takes; and the sizes the mixers' own arithmetic is priced with."""
+    from minivllm_amd.models.causal_lm import expected_tensors
+    ex = llm.executor
+    decls = expected_tensors(ex.arch, cfg, ex.plan)
+    params = sum(_numel(d.shape) for d in decls.values())
+    expert = sum(_numel(d.shape) for n, d in decls.items() if ".mlp.e" in n)
+    matrices = sum(_numel(d.shape) for n, d in decls.items() if len(d.shape) == 2 and n != "embed" and ".mlp.e" not in n
+                   and not n.endswith(".conv"))
+    routers = [(l.mlp.experts, l.mlp.top) for l in cfg.layers if l.mlp is not None and l.mlp.kind == "moe"]
+    per_layer_expert = expert // max(1, len(routers))
+    active = sum(per_layer_expert * min(t, e) // max(e, 1) for e, t in routers)
+    state_bytes = sum(t[0].numel() * t.element_size() for ts in ex.state_tensors.values() for t in ts.values())
+    kv_bytes = sum(need.bytes_per_token(ex.dtype) for need in ex.needs if need is not None)
+    attn = [(l.mixer.heads, l.mixer.kv_rank, l.mixer.rot_dim, l.mixer.dim, l.mixer.vdim) for l in cfg.layers
+            if l.mixer.type == "latent_attention"]
+    states = [(l.mixer.heads, l.mixer.dim, l.mixer.vdim + (l.mixer.type == "mlstm"), 6 if l.mixer.type == "delta" else 4)
+              for l in cfg.layers if l.mixer.type != "latent_attention"]
+    return dict(params=params, matrices=matrices, expert=expert, active=active, routers=routers,
+                per_layer_expert=per_layer_expert, state_bytes=state_bytes, kv_bytes=kv_bytes, attn=attn, states=states)
+
+
+def bench_dutilix(args, llm, cfg, layers, layers_full, item) -> int:
+    """The default measurements for a Dutilix model of the named shape; the same fields in the line."""
+    nums = dutilix_numbers(llm, cfg, item)
+    prefill = None
+    if args.only in ("all", "prefill"):
+        prefill_s = measure_prefill(llm, cfg.vocab_size, args.prefill_tokens, repeats=3, seed=args.seed)
+        T = args.prefill_tokens
+        flops = 2 * T * (nums["matrices"] + nums["active"] - cfg.vocab_size * cfg.hidden_size) + 2 * cfg.vocab_size * cfg.hidden_size
+        for H, R, dr, dn, dv in nums["attn"]:
+            # as the engine computes it: queries carried into the latent's space, scores and sums over the latents
+            flops += 2 * T * H * (dn + dv) * R + 2 * H * (2 * R + dr) * T * (T + 1) // 2
+        for H, dk, cols, per in nums["states"]:
+            flops += per * T * H * dk * cols
+        prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+                   "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+    tok_s = ms_step = roofline = None
+    ran = regions = 0
+    if args.only in ("all", "decode"):
+        tok_s, ms_step, mean_ctx, ran, regions = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len,
+                                                                args.steps, args.warmup, args.seed)
+        # every weight that some request of the step uses once (of a layer's E experts about E (1 - (1 - top/E)^batch)),
+        # each request's states read and written, its cached latents read
+        touched = sum(nums["per_layer_expert"] * (1.0 - (1.0 - min(t, e) / e) ** args.batch) for e, t in nums["routers"])
+        step_bytes = (nums["params"] - nums["expert"] + touched) * item + args.batch * (2 * nums["state_bytes"] + mean_ctx * nums["kv_bytes"])
+        achieved = step_bytes / (ms_step * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(achieved / PEAK_HBM_GBS, 4)}
+    points = {}
+    if not args.no_points and args.only == "all":
+        for b, key in ((1, "decode_b1"), (64, "decode_b64")):
+            n = min(args.steps, 128)
+            points[key] = round(measure_decode(llm, cfg.vocab_size, b, args.prompt_len, n, min(args.warmup, 8),
+                                               args.seed + b)[0], 1)
+    kinds = [l.mixer.type for l in cfg.layers]
+    config = {"model": f"dutilix-{args.shape}-shape-random", "layers": layers, "layers_full": layers_full,
+              "hidden": cfg.hidden_size, "vocab": cfg.vocab_size, "delta_layers": kinds.count("delta"),
+              "mlstm_layers": kinds.count("mlstm"), "latent_attention_layers": kinds.count("latent_attention"),
+              "moe_layers": len(nums["routers"]), "experts": args.experts, "top": args.top, "weights": nums["params"],
+              "weights_a_token_uses": nums["params"] - nums["expert"] + nums["active"], "global_batch": args.batch,
+              "seq_len": args.context, "prompt_len": args.prompt_len, "block_size": args.block_size, "graph": not args.no_graph,
+              "scheduler_steps": args.scheduler_steps, "launch_ahead": bool(llm.config.launch_ahead),
+              "parallelism": "single-gpu"}
+    print(json.dumps({"metric": "decode tok/s (batch %d, %d-token prompts)" % (args.batch, args.prompt_len),
+                      "value": round(tok_s, 1) if tok_s is not None else None, "unit": "tokens/s", "n_gpus": 1,
+                      "steps": ran if ran else args.steps, "warmup": args.warmup,
+                      "ms_per_step": round(ms_step, 4) if ms_step is not None else None, "higher_is_better": True,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                      "data": "synthetic", "config": config, "timed_regions": regions, "prefill": prefill,
+                      "roofline": roofline, "points": points}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--shape", choices=sorted(SHAPES), default="0.6b")
-    ap.add_argument("--design", choices=["qwen3", "bolapel"], default="qwen3",
+    ap.add_argument("--experts", type=int, default=32, help="--design dutilix: experts of each mixture layer")
+    ap.add_argument("--top", type=int, default=4, help="--design dutilix: experts a token uses (each 1/top of the dense width)")
+    ap.add_argument("--design", choices=["qwen3", "bolapel", "dutilix"], default="qwen3",
                     help="'bolapel': the same widths, head counts, vocabulary and number of layers as the named Qwen3 "
                          "shape, as a Bolapel model (three delta-rule layers to one attention layer in chunks of --chunk "
                          "tokens); decode and prefill are measured the same way and the line names the design")
@@ -468,6 +549,8 @@ def main() -> int:
     item = 2 if args.dtype == "bfloat16" else 4
     if args.design == "bolapel":
         return bench_bolapel(args, llm, cfg, layers, layers_full, item)
+    if args.design == "dutilix":
+        return bench_dutilix(args, llm, cfg, layers, layers_full, item)
     nums = model_numbers(shape, layers)
 
     prefill = None

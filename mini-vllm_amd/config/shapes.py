@@ -27,9 +27,11 @@ def named_shapes() -> Dict[str, Dict[str, Any]]:
     added here."""
     shapes = {name: qwen3_shape(name) for name in QWEN3_SHAPES}
     shapes["bolapel-tiny"] = bolapel_tiny_shape()
+    shapes["dutilix-tiny"] = dutilix_tiny_shape()
     for name in QWEN3_SHAPES:
         if name != "tiny":
             shapes[f"bolapel-{name}"] = bolapel_shape(name)
+            shapes[f"dutilix-{name}"] = dutilix_shape(name)
     return shapes
 
 
@@ -88,3 +90,48 @@ def bolapel_tiny_shape() -> Dict[str, Any]:
                        {"type": "attention", "mixer": dict(attn), "mlp": ff},
                        {"type": "general_delta", "mixer": {"heads": 4, "dim": 8, "rank": 8}, "mlp": None},
                        {"type": "attention", "mixer": dict(attn, kv_from=1), "mlp": ff}]}
+
+
+def dutilix_shape(name: str, layers: int = None, experts: int = 32, top: int = 4, identity: int = 0, groups: int = 4,
+                  keep: int = 2, state_head_dim: int = 64, kv_rank: int = 256, rot_dim: int = 64, conv: int = 4,
+                  pattern: int = 4) -> Dict[str, Any]:
+    """A Dutilix configuration with the width, vocabulary, head count, head size and number of layers of the
+    named Qwen3 shape: every ``pattern``-th layer is attention over a cached latent of ``kv_rank`` numbers (a
+    rotated key part of ``rot_dim``), the others alternate between the gated delta rule (a query/key group for
+    every two heads) and the mLSTM, both with heads of ``state_head_dim``. Every second feed-forward is a mixture
+    of ``experts`` experts of which ``top`` are used, each 1/top of the shape's dense width, the others are dense.
+    For random-weights models at sizes that resemble a real model's layers."""
+    q = QWEN3_SHAPES[name]
+    n = layers or q["num_hidden_layers"]
+    hid, hd, heads = q["hidden_size"], q["head_dim"], q["num_attention_heads"]
+    state_heads = hid // state_head_dim
+    dense = {"kind": "dense", "ff": q["intermediate_size"]}
+    sparse = {"kind": "moe", "expert": {"ff": q["intermediate_size"] // top},
+              "router": {"experts": experts, "identity": identity, "top": top, "groups": {"count": groups, "keep": keep}}}
+    out = []
+    for i in range(n):
+        mlp = sparse if i % 2 else dense
+        if i % pattern == pattern - 1:
+            m = {"heads": heads, "dim": hd, "rot_dim": rot_dim, "vdim": hd, "q_rank": max(64, hid // 4), "kv_rank": kv_rank,
+                 "scale": (hd + rot_dim) ** -0.5, "rot": {"dims": rot_dim, "base": q["rope_theta"]}}
+            out.append({"type": "latent_attention", "mixer": m, "mlp": mlp})
+        elif i % 2 == 0:
+            out.append({"type": "delta", "mlp": mlp, "mixer": {"heads": state_heads, "kv_heads": max(1, state_heads // 2),
+                                                               "dim": state_head_dim, "vdim": state_head_dim, "conv": conv}})
+        else:
+            out.append({"type": "mlstm", "mlp": mlp, "mixer": {"heads": state_heads, "dim": state_head_dim,
+                                                               "vdim": state_head_dim, "gate_cap": 15.0}})
+    return {"architecture": "Dutilix", "vocab": q["vocab_size"], "width": hid, "layers": out,
+            "norm": {"eps": q["rms_norm_eps"]}, "logit_scale": 1.0}
+
+
+def dutilix_tiny_shape() -> Dict[str, Any]:
+    """A Dutilix model of a few thousand weights with every kind of layer and feed-forward."""
+    moe = {"kind": "moe", "expert": {"ff": 32},
+           "router": {"experts": 6, "identity": 2, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    return {"architecture": "Dutilix", "vocab": 256, "width": 64, "norm": {"eps": 1e-5}, "logit_scale": 0.5,
+            "layers": [{"type": "delta", "mixer": {"heads": 4, "kv_heads": 2, "dim": 8, "vdim": 16, "conv": 3}, "mlp": moe},
+                       {"type": "latent_attention", "mlp": {"kind": "dense", "ff": 96},
+                        "mixer": {"heads": 4, "dim": 12, "rot_dim": 4, "vdim": 8, "q_rank": 24, "kv_rank": 16, "scale": 0.25,
+                                  "rot": {"dims": 4, "base": 10000.0}}},
+                       {"type": "mlstm", "mixer": {"heads": 2, "dim": 16, "vdim": 24, "gate_cap": 12.0}, "mlp": None}]}

@@ -63,23 +63,25 @@ def gated_delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: t
 
 
 def delta_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, m: dict, eps: float,
-                state: Optional[dict] = None) -> Tuple[torch.Tensor, dict]:
-    H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+                state: Optional[dict] = None, rnd=None) -> Tuple[torch.Tensor, dict]:
+    """``rnd`` rounds what an engine with 16-bit activations would store (projections, the gated output)."""
+    rnd = rnd or (lambda t: t)
+    H, G, dk, dv = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"]
     n = h.shape[0]
     state = state or {}
     new = {}
     proj = {}
     for name in ("q", "k", "v"):
-        y, new["conv." + name] = short_conv(h @ w[prefix + name].T, w[prefix + name + ".conv"], state.get("conv." + name))
+        y, new["conv." + name] = short_conv(rnd(h @ w[prefix + name].T), w[prefix + name + ".conv"], state.get("conv." + name))
         proj[name] = silu(y)
     q = proj["q"].view(n, G, dk)
     k = proj["k"].view(n, G, dk)
     v = proj["v"].view(n, H, dv)
     q = q / torch.sqrt(q.pow(2).sum(-1, keepdim=True) + UNIT_EPS) * dk ** -0.5
     k = k / torch.sqrt(k.pow(2).sum(-1, keepdim=True) + UNIT_EPS)
-    beta = torch.sigmoid(h @ w[prefix + "b"].T)                                       # [n, H]
-    decay = torch.exp(-torch.exp(w[prefix + "A_log"]) * torch.nn.functional.softplus(h @ w[prefix + "a"].T + w[prefix + "dt_bias"]))
-    gate = silu(h @ w[prefix + "g"].T).view(n, H, dv)
+    beta = torch.sigmoid(rnd(h @ w[prefix + "b"].T))                                  # [n, H]
+    decay = torch.exp(-torch.exp(w[prefix + "A_log"]) * torch.nn.functional.softplus(rnd(h @ w[prefix + "a"].T) + w[prefix + "dt_bias"]))
+    gate = silu(rnd(h @ w[prefix + "g"].T)).view(n, H, dv)
     out = torch.empty(n, H, dv, dtype=h.dtype)
     states = []
     for head in range(H):
@@ -89,8 +91,8 @@ def delta_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, m: dic
         out[:, head] = o
         states.append(S)
     new["S"] = torch.stack(states)
-    out = rms_norm(out, w[prefix + "norm"], eps) * gate
-    return out.reshape(n, H * dv) @ w[prefix + "o"].T, new
+    out = rnd(rms_norm(out, w[prefix + "norm"], eps) * gate)
+    return rnd(out.reshape(n, H * dv) @ w[prefix + "o"].T), new
 
 
 # ---------------------------------------------------------------------------------------
@@ -119,14 +121,15 @@ def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, log_in: torch.
 
 
 def mlstm_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, m: dict, eps: float,
-                state: Optional[dict] = None) -> Tuple[torch.Tensor, dict]:
+                state: Optional[dict] = None, rnd=None) -> Tuple[torch.Tensor, dict]:
+    rnd = rnd or (lambda t: t)
     H, dk, dv, cap = m["heads"], m["dim"], m["vdim"], float(m["gate_cap"])
     n = h.shape[0]
-    q = (h @ w[prefix + "q"].T * dk ** -0.5).view(n, H, dk)
-    k = (h @ w[prefix + "k"].T).view(n, H, dk)
-    v = (h @ w[prefix + "v"].T).view(n, H, dv)
-    log_in = cap * torch.tanh((h @ w[prefix + "i"].T + w[prefix + "i.b"]) / cap)
-    log_forget = torch.nn.functional.logsigmoid(cap * torch.tanh((h @ w[prefix + "f"].T + w[prefix + "f.b"]) / cap))
+    q = (rnd(h @ w[prefix + "q"].T) * dk ** -0.5).view(n, H, dk)
+    k = rnd(h @ w[prefix + "k"].T).view(n, H, dk)
+    v = rnd(h @ w[prefix + "v"].T).view(n, H, dv)
+    log_in = cap * torch.tanh((rnd(h @ w[prefix + "i"].T) + w[prefix + "i.b"]) / cap)
+    log_forget = torch.nn.functional.logsigmoid(cap * torch.tanh((rnd(h @ w[prefix + "f"].T) + w[prefix + "f.b"]) / cap))
     out = torch.empty(n, H, dv, dtype=h.dtype)
     new = []
     for head in range(H):
@@ -134,8 +137,8 @@ def mlstm_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, m: dic
                            None if state is None else state["heads"][head])
         out[:, head] = o
         new.append(st)
-    out = rms_norm(out, None, eps).reshape(n, H * dv) * w[prefix + "norm"] * torch.sigmoid(h @ w[prefix + "g"].T)
-    return out @ w[prefix + "o"].T, {"heads": new}
+    out = rnd(rms_norm(out, None, eps).reshape(n, H * dv) * w[prefix + "norm"] * torch.sigmoid(rnd(h @ w[prefix + "g"].T)))
+    return rnd(out @ w[prefix + "o"].T), {"heads": new}
 
 
 # ---------------------------------------------------------------------------------------
@@ -155,18 +158,20 @@ def rotate_half_layout(x: torch.Tensor, positions: torch.Tensor, dims: int, base
 
 def latent_attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, m: dict, eps: float,
                            positions: Optional[torch.Tensor] = None,
-                           cache: Optional[tuple] = None) -> Tuple[torch.Tensor, tuple]:
+                           cache: Optional[tuple] = None, rnd=None) -> Tuple[torch.Tensor, tuple]:
     """``cache`` = (latents [j, kv_rank], rotated key parts [j, rot_dim]) of the tokens in front."""
-    H, dn, dr, dv, rank = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+    rnd = rnd or (lambda t: t)
+    H, dn, dr, dv, rank = m["heads"], m["dim"], m.get("rot_dim", 0), m["vdim"], m["kv_rank"]
     n = h.shape[0]
     start = 0 if cache is None else cache[0].shape[0]
     pos = torch.arange(start, start + n) if positions is None else positions
-    cq = rms_norm(h @ w[prefix + "dq"].T, w[prefix + "dq.norm"], eps)
-    q = (cq @ w[prefix + "uq"].T).view(n, H, dn + dr)
-    q_plain, q_rot = q[..., :dn], rotate_half_layout(q[..., dn:], pos, m["rot"]["dims"], m["rot"]["base"])
-    down = h @ w[prefix + "dkv"].T
-    lat = rms_norm(down[:, :rank], w[prefix + "dkv.norm"], eps)
-    k_rot = rotate_half_layout(down[:, rank:], pos, m["rot"]["dims"], m["rot"]["base"])
+    rot = (lambda x: rotate_half_layout(x, pos, m["rot"]["dims"], m["rot"]["base"])) if dr else (lambda x: x)
+    cq = rnd(rms_norm(rnd(h @ w[prefix + "dq"].T), w[prefix + "dq.norm"], eps))
+    q = rnd(cq @ w[prefix + "uq"].T).view(n, H, dn + dr)
+    q_plain, q_rot = q[..., :dn], rot(q[..., dn:])
+    down = rnd(h @ w[prefix + "dkv"].T)
+    lat = rnd(rms_norm(down[:, :rank], w[prefix + "dkv.norm"], eps))
+    k_rot = rnd(rot(down[:, rank:]))
     if cache is not None:
         lat, k_rot = torch.cat([cache[0], lat]), torch.cat([cache[1], k_rot])
     total = lat.shape[0]
@@ -176,15 +181,16 @@ def latent_attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: 
     visible = torch.arange(total)[None, :] <= pos[:, None]
     score = score.masked_fill(~visible[None], float("-inf"))
     out = torch.einsum("hij,jhd->ihd", torch.softmax(score, dim=-1), val).reshape(n, H * dv)
-    out = out * torch.sigmoid(h @ w[prefix + "g"].T)
-    return out @ w[prefix + "o"].T, (lat, k_rot)
+    out = rnd(out * torch.sigmoid(rnd(h @ w[prefix + "g"].T)))
+    return rnd(out @ w[prefix + "o"].T), (lat, k_rot)
 
 
 # ---------------------------------------------------------------------------------------
 # feed-forwards
 # ---------------------------------------------------------------------------------------
-def gated_pair(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
-    return (silu(h @ gate.T) * (h @ up.T)) @ down.T
+def gated_pair(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, rnd=None) -> torch.Tensor:
+    rnd = rnd or (lambda t: t)
+    return (rnd(silu(rnd(h @ gate.T)) * rnd(h @ up.T))) @ down.T
 
 
 def route(h: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int):
@@ -204,11 +210,11 @@ def route(h: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top: 
     return chosen, picked / (picked.sum(-1, keepdim=True) + WEIGHT_SUM_EPS)
 
 
-def mixture(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, mlp: dict) -> torch.Tensor:
+def mixture(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, mlp: dict, rnd=None) -> torch.Tensor:
     r = mlp["router"]
     real = r["experts"]
-    chosen, weight = route(h, w[prefix + "router"], w[prefix + "correction"], r["top"], r["groups"]["count"],
-                           r["groups"]["keep"])
+    groups = r.get("groups") or {"count": 1, "keep": 1}
+    chosen, weight = route(h, w[prefix + "router"], w[prefix + "correction"], r["top"], groups["count"], groups["keep"])
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, a in zip(chosen[t].tolist(), weight[t]):
@@ -216,15 +222,15 @@ def mixture(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, mlp: dict)
                 out[t] += a * h[t]
             else:
                 p = f"{prefix}e{e}."
-                out[t] += a * gated_pair(h[t:t + 1], w[p + "gate"], w[p + "up"], w[p + "down"])[0]
+                out[t] += a * gated_pair(h[t:t + 1], w[p + "gate"], w[p + "up"], w[p + "down"], rnd)[0]
     return out
 
 
-def feed_forward(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, mlp: dict) -> torch.Tensor:
+def feed_forward(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, mlp: dict, rnd=None) -> torch.Tensor:
     if mlp["kind"] == "dense":
-        return gated_pair(h, w[prefix + "gate"], w[prefix + "up"], w[prefix + "down"])
+        return gated_pair(h, w[prefix + "gate"], w[prefix + "up"], w[prefix + "down"], rnd)
     if mlp["kind"] == "moe":
-        return mixture(h, w, prefix, mlp)
+        return mixture(h, w, prefix, mlp, rnd)
     raise ValueError(mlp["kind"])
 
 
@@ -234,27 +240,33 @@ def feed_forward(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, mlp: 
 MIXERS = {"delta": delta_mixer, "mlstm": mlstm_mixer}
 
 
+def round_to_bfloat16(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
 def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], states: Optional[list] = None,
-            return_layers: bool = False):
+            return_layers: bool = False, rnd=None):
     """Logits [n, vocab] of ``tokens`` continuing a sequence whose per-layer ``states`` are given (None at
-    the start). Returns (logits, new states[, residual stream after every layer])."""
+    the start). Returns (logits, new states[, residual stream after every layer]). ``rnd`` rounds what an
+    engine with 16-bit activations would store; the residual stream stays as it is."""
+    rnd = rnd or (lambda t: t)
     eps = cfg["norm"]["eps"]
     x = w["embed"][torch.tensor(tokens, dtype=torch.long)]
     states = states or [None] * len(cfg["layers"])
     new_states, streams = [], []
     for i, layer in enumerate(cfg["layers"]):
         p = f"l{i}."
-        hin = rms_norm(x, w[p + "norm1"], eps)
+        hin = rnd(rms_norm(x, w[p + "norm1"], eps))
         if layer["type"] == "latent_attention":
-            y, st = latent_attention_mixer(hin, w, p + "mix.", layer["mixer"], eps, cache=states[i])
+            y, st = latent_attention_mixer(hin, w, p + "mix.", layer["mixer"], eps, cache=states[i], rnd=rnd)
         else:
-            y, st = MIXERS[layer["type"]](hin, w, p + "mix.", layer["mixer"], eps, states[i])
+            y, st = MIXERS[layer["type"]](hin, w, p + "mix.", layer["mixer"], eps, states[i], rnd=rnd)
         new_states.append(st)
         x = x + y
         if layer.get("mlp") is not None:
-            x = x + feed_forward(rms_norm(x, w[p + "norm2"], eps), w, p + "mlp.", layer["mlp"])
+            x = x + rnd(feed_forward(rnd(rms_norm(x, w[p + "norm2"], eps)), w, p + "mlp.", layer["mlp"], rnd))
         streams.append(x)
-    logits = rms_norm(x, w["final.norm"], eps) @ w["head"].T * cfg.get("logit_scale", 1.0)
+    logits = rnd(rms_norm(x, w["final.norm"], eps)) @ w["head"].T * cfg.get("logit_scale", 1.0)
     if return_layers:
         return logits, new_states, torch.stack(streams)
     return logits, new_states
