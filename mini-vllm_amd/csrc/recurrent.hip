@@ -778,8 +778,8 @@ extern "C" int mv_gdelta_prepare(const void* packed, long ld, int n, int n_seqs,
 // input gate i = cap tanh((i + i_bias) / cap), the log forget gate f = logsigmoid(cap tanh((f + f_bias) / cap))
 // and the running maximum m (kept per request and head, 0 at the start):
 //     m' = max(f + m, i);   a = exp(f + m - m');   b = exp(i - m');   gates = (a, b, exp(-m'), 0)
-// One wave per (request, head) walks the request's rows 64 at a time: m' is a scan with the
-// associative step (F, I) after (F0, I0) = (F0 + F, max(I0 + F, I)), m' = max(F + m, I).
+// One wave per (request, head) walks the request's rows 64 at a time: the gates' functions are computed
+// a row a lane, the maximum itself in the order of the rows.
 // ---------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(64)
@@ -798,17 +798,19 @@ mlstm_gates_kernel(const T* __restrict__ packed, long ld, int H, long gate_off, 
         const T* p = packed + (size_t)(live ? t : first) * ld + gate_off;
         const float gi = cap * tanhf((to_f(p[head]) + bi) / cap);
         const float gf = logsigmoid_f(cap * tanhf((to_f(p[H + head]) + bf) / cap));
-        float F = live ? gf : 0.f, I = live ? gi : -INFINITY;         // rows past the end change nothing
-        for (int o = 1; o < 64; o <<= 1) {
-            const float Fp = __shfl_up(F, o, 64), Ip = __shfl_up(I, o, 64);
-            if (lane >= o) {
-                I = fmaxf(Ip + F, I);
-                F = Fp + F;
+        // the maximum runs token by token, in the same order however the request was cut into steps: every lane
+        // walks the 64 rows (their gates come by lane broadcasts), lane j keeps the values of row j
+        float m_prev = m, m_new = m;
+        const int nt = min(64, end - base);
+        for (int j = 0; j < nt; ++j) {
+            const float fj = __shfl(gf, j, 64), ij = __shfl(gi, j, 64);
+            const float next = fmaxf(fj + m, ij);
+            if (lane == j) {
+                m_prev = m;
+                m_new = next;
             }
+            m = next;
         }
-        const float m_new = fmaxf(F + m, I);
-        float m_prev = __shfl_up(m_new, 1, 64);
-        if (lane == 0) m_prev = m;
         if (live) {
             float* g = gates + ((size_t)t * H + head) * 4;
             g[0] = expf(gf + m_prev - m_new);
@@ -816,7 +818,6 @@ mlstm_gates_kernel(const T* __restrict__ packed, long ld, int H, long gate_off, 
             g[2] = expf(-m_new);
             g[3] = 0.f;
         }
-        m = __shfl(m_new, 63, 64);
     }
     if (lane == 0) *ms = m;
 }

@@ -268,8 +268,8 @@ def test_mlstm_steps_and_states(dtype, H, dk, dv, cap):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_mlstm_one_by_one_against_the_prompt(dtype):
-    """100 tokens in one step and one by one: the outputs agree to rounding (the gate scan adds the forget gates in
-    another order), and the decoded rows agree with the plain scan."""
+    """100 tokens in one step and one by one: the same bits (the running maximum is taken in the order of the tokens
+    however they are cut), and the rows agree with the plain scan."""
     ops = ops_for(dtype)
     H, dk, dv, cap, eps, n = 2, 16, 12, 6.0, 1e-6, 100
     packed, t = mlstm_setup(H, dk, dv, n, seed=3, dtype=dtype)
@@ -282,7 +282,7 @@ def test_mlstm_one_by_one_against_the_prompt(dtype):
             rows.append(run_mlstm(ops, packed[base:base + c], t, H, dk, dv, cap, eps, state, maxima, [c], [0]).clone())
             base += c
         outs.append(torch.cat(rows))
-    close(outs[1], outs[0].double(), 1e-5 if dtype == torch.float32 else 8e-3, "one by one against whole")
+    assert torch.equal(outs[1], outs[0]), "one by one against whole"
     close(outs[1], mlstm_plain(packed, t, H, dk, dv, cap, eps, [None] * H)[1], 3e-5 if dtype == torch.float32 else 1.2e-2, "plain")
 
 
@@ -378,10 +378,9 @@ def test_latent_attention_prompt_and_continuation(dtype, H, dn, dr, dv, qr, R, p
     w, h = latent_case(H, dn, dr, dv, qr, R, seed=H + dn, dtype=dtype, n=n_a + n_b, key_gain=2.0)
     ha, hb = h[:n_a], h[n_a:]
     w64 = {"x." + k: v.double() for k, v in w.items()}
-    rnd = None if dtype == torch.float32 else plain.round_to_bfloat16
     want_a = plain.latent_attention_mixer(ha.double(), w64, "x.", m, eps, rnd=None)[0]
     want_b = plain.latent_attention_mixer(hb.double(), w64, "x.", m, eps, rnd=None)[0]
-    tol = 3e-5 if dtype == torch.float32 else 2.5e-2
+    tol = 3e-5 if dtype == torch.float32 else 5e-2          # (single rows of a steep softmax, relative to the row's own largest value)
     n_pages = 64 if page_size == 16 else 256
     pages = torch.full((n_pages, page_size, R + dr), float("nan"), dtype=dtype, device=DEV)
     perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(5)).tolist()
