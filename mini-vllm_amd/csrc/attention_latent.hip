@@ -84,20 +84,25 @@ extern "C" int mv_latent_prepare(const void* packed, long ld, int n, int QR, int
 // Per-head linear map. x rows [n][H][ldx_head] (IN inputs used), w [H][IN][OUT] (the inputs of an
 // output column are a stride of OUT apart, so neighbouring threads read neighbouring words),
 // y rows [n][H][ldy_head]:  y[t][h][j] = sum_i x[t][h][i] w[h][i][j], the sum in the order of i.
-// A workgroup takes HL_TOKENS rows of one head; the weight is read once for them.
 //   tail > 0   x[t][h][IN .. IN+tail) is copied behind the OUT outputs, rotated by the row's position
 //              (pairs i, i + tail/2; table[p] = [cos | sin])
 //   gate       y is multiplied by sigmoid(gate[t][h * OUT + j])
 // ---------------------------------------------------------------------------------------
 #define HL_TOKENS 8
 #define HL_MAX_IN 1024
+#define HL_COLS 64
+#define HL_SLICES 4
 
+// A workgroup takes HL_TOKENS rows, one head and HL_COLS output columns; its 256 threads are HL_COLS columns
+// times HL_SLICES slices of the inputs (slice s sums inputs s, s + HL_SLICES, ...), the slices are added in
+// order through LDS. The order of additions depends on IN alone.
 template <typename TIN, typename TOUT, typename TG>
 __global__ void __launch_bounds__(256)
 head_linear_kernel(const TIN* __restrict__ x, long ldx, int ldx_head, WeightPtr w, int IN, int OUT, TOUT* __restrict__ y, long ldy,
                    int ldy_head, int tail, const float* __restrict__ table, const int* __restrict__ positions,
                    const TG* __restrict__ gate, long ldg, const int* __restrict__ token_seq, int n) {
     __shared__ float xs[HL_TOKENS][HL_MAX_IN];
+    __shared__ float part[HL_SLICES][HL_TOKENS][HL_COLS];
     const int t0 = blockIdx.x * HL_TOKENS, head = blockIdx.y, tid = threadIdx.x;
     const int nt = min(HL_TOKENS, n - t0);
     for (int e = tid; e < HL_TOKENS * IN; e += 256) {
@@ -105,26 +110,44 @@ head_linear_kernel(const TIN* __restrict__ x, long ldx, int ldx_head, WeightPtr 
         xs[tt][i] = tt < nt ? to_f(x[(size_t)(t0 + tt) * ldx + (size_t)head * ldx_head + i]) : 0.f;
     }
     __syncthreads();
-    for (int j = tid; j < OUT; j += 256) {
-        float acc[HL_TOKENS];
+    const int col = tid % HL_COLS, slice = tid / HL_COLS;
+    const int j = blockIdx.z * HL_COLS + col;
+    float acc[HL_TOKENS];
 #pragma unroll
-        for (int tt = 0; tt < HL_TOKENS; ++tt) acc[tt] = 0.f;
+    for (int tt = 0; tt < HL_TOKENS; ++tt) acc[tt] = 0.f;
+    if (j < OUT) {
         const size_t w0 = (size_t)head * IN * OUT + j;
-        for (int i = 0; i < IN; ++i) {
+        int i = slice;
+        for (; i + 3 * HL_SLICES < IN; i += 4 * HL_SLICES) {          // four loads in flight
+            float wv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) wv[u] = w.at(w0 + (size_t)(i + u * HL_SLICES) * OUT);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int tt = 0; tt < HL_TOKENS; ++tt) acc[tt] = fmaf(xs[tt][i + u * HL_SLICES], wv[u], acc[tt]);
+        }
+        for (; i < IN; i += HL_SLICES) {
             const float wv = w.at(w0 + (size_t)i * OUT);
 #pragma unroll
             for (int tt = 0; tt < HL_TOKENS; ++tt) acc[tt] = fmaf(xs[tt][i], wv, acc[tt]);
         }
-#pragma unroll
-        for (int tt = 0; tt < HL_TOKENS; ++tt) {
-            if (tt < nt) {
-                float v = acc[tt];
-                if (token_seq[t0 + tt] < 0) v = 0.f;
-                else if (gate) v *= 1.f / (1.f + expf(-to_f(gate[(size_t)(t0 + tt) * ldg + (size_t)head * OUT + j])));
-                y[(size_t)(t0 + tt) * ldy + (size_t)head * ldy_head + j] = from_f<TOUT>(v);
-            }
-        }
     }
+#pragma unroll
+    for (int tt = 0; tt < HL_TOKENS; ++tt) part[slice][tt][col] = acc[tt];
+    __syncthreads();
+    for (int e = tid; e < nt * HL_COLS; e += 256) {
+        const int tt = e / HL_COLS, c = e % HL_COLS;
+        const int jj = blockIdx.z * HL_COLS + c;
+        if (jj >= OUT) continue;
+        float v = 0.f;
+#pragma unroll
+        for (int sl = 0; sl < HL_SLICES; ++sl) v += part[sl][tt][c];
+        if (token_seq[t0 + tt] < 0) v = 0.f;
+        else if (gate) v *= 1.f / (1.f + expf(-to_f(gate[(size_t)(t0 + tt) * ldg + (size_t)head * OUT + jj])));
+        y[(size_t)(t0 + tt) * ldy + (size_t)head * ldy_head + jj] = from_f<TOUT>(v);
+    }
+    if (blockIdx.z != 0) return;
     const int half = tail / 2;
     for (int e = tid; e < nt * half; e += 256) {
         const int tt = e / half, i = e % half;
@@ -157,7 +180,7 @@ extern "C" int mv_head_linear(const void* x, long ldx, int ldx_head, const void*
     MV_REQUIRE((mode == 0 && !gate) || (mode == 1 && tail == 0), "head_linear: mode %d does not take these options", mode);
     if (n == 0) return 0;
     WeightPtr wp{w, weight_dtype};
-    dim3 grid((n + HL_TOKENS - 1) / HL_TOKENS, H);
+    dim3 grid((n + HL_TOKENS - 1) / HL_TOKENS, H, (OUT + HL_COLS - 1) / HL_COLS);
     if (mode == 0) {
         MV_DISPATCH_T(dtype, "head_linear",
                       hipLaunchKernelGGL((head_linear_kernel<T, float, T>), grid, dim3(256), 0, stream, (const T*)x, ldx, ldx_head,
@@ -298,4 +321,233 @@ extern "C" int mv_attention_latent(const float* q, long ldq, float* out, long ld
                                      stream, q, ldq, out, ldo, (const T*)pages, block_table, bt_width, page_size, positions,
                                      token_seq, H, R, DR, scale));
     return mv_check_launch("attention_latent");
+}
+
+// ---------------------------------------------------------------------------------------
+// Attention for steps of few rows (single decoded tokens): a row's keys are dealt out to workgroups in
+// runs of ALS_SPLIT positions (run s holds positions s * ALS_SPLIT ..., so the cutting depends on the
+// position alone), a workgroup serves up to ALS_HEADS heads of the row at once and brings each tile of
+// ALS_TILE key rows into LDS with 16-byte loads, where all its heads read them. It leaves per run the
+// running maximum, the sum of weights and the weighted sum of latents; a second kernel joins the runs
+// in their order. Requires (R + DR) * sizeof(T) to be a multiple of 16.
+// ---------------------------------------------------------------------------------------
+#define ALS_SPLIT 256
+#define ALS_TILE 32
+#define ALS_HEADS 16
+#define ALS_THREADS 256
+
+template <typename T> struct AlsWord;
+template <> struct AlsWord<float> { static constexpr int per = 1; };
+template <> struct AlsWord<bf16> { static constexpr int per = 2; };
+
+template <typename T>
+__device__ __forceinline__ void als_unpack(uint32_t w, float (&out)[AlsWord<T>::per]) {
+    if constexpr (AlsWord<T>::per == 1) {
+        out[0] = __uint_as_float(w);
+    } else {
+        out[0] = __uint_as_float(w << 16);
+        out[1] = __uint_as_float(w & 0xffff0000u);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(ALS_THREADS)
+attention_latent_split_kernel(const float* __restrict__ q, long ldq, const T* __restrict__ pages, const int* __restrict__ block_table,
+                              int bt_width, int page_size, const int* __restrict__ positions, const int* __restrict__ token_seq,
+                              int H, int R, int DR, float scale, int row_words, int max_splits, float* __restrict__ part_o,
+                              float* __restrict__ part_ml) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char als_lds[];
+    constexpr int PER = AlsWord<T>::per;
+    const int DK = R + DR;
+    const int words = DK / PER;                             // words of a key row; row_words (odd) is its pitch in LDS
+    float* qs = reinterpret_cast<float*>(als_lds);          // [ALS_HEADS][DK]
+    uint32_t* tile = reinterpret_cast<uint32_t*>(qs + ALS_HEADS * DK);      // [ALS_TILE][row_words]
+    float* ps = reinterpret_cast<float*>(tile + ALS_TILE * row_words);      // [ALS_TILE][ALS_HEADS]
+    float* cs = ps + ALS_TILE * ALS_HEADS;                  // [ALS_HEADS]
+    const int tok = blockIdx.x, h0 = blockIdx.y * ALS_HEADS, split = blockIdx.z, tid = threadIdx.x;
+    const int seq = token_seq[tok];
+    if (seq < 0) return;
+    const int pos = positions[tok];
+    const int lo = split * ALS_SPLIT;
+    if (lo > pos) return;
+    const int hi = min(pos, lo + ALS_SPLIT - 1);
+    const int nh = min(ALS_HEADS, H - h0);
+    const int* bt = block_table + (size_t)seq * bt_width;
+    for (int e = tid; e < ALS_HEADS * DK; e += ALS_THREADS) {
+        const int hh = e / DK, d = e % DK;
+        qs[e] = hh < nh ? q[(size_t)tok * ldq + (size_t)(h0 + hh) * DK + d] * scale : 0.f;
+    }
+    // scores: thread (key j of the tile, head pair hp) -> heads 2 hp, 2 hp + 1; sums: thread -> latent channels tid, tid + 256
+    const int j = tid % ALS_TILE, hp = tid / ALS_TILE;
+    float m0 = -INFINITY, m1 = -INFINITY, l0 = 0.f, l1 = 0.f;
+    float acc[2][ALS_HEADS];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int hh = 0; hh < ALS_HEADS; ++hh) acc[c][hh] = 0.f;
+    const int vec_per_row = words / 4;                      // 16-byte pieces of a key row
+    for (int base = lo; base <= hi; base += ALS_TILE) {
+        const int cnt = min(ALS_TILE, hi - base + 1);
+        __syncthreads();                                    // the tile before has been read (and qs is written)
+        for (int e = tid; e < cnt * vec_per_row; e += ALS_THREADS) {
+            const int jj = e / vec_per_row, v = e % vec_per_row;
+            const int p = base + jj;
+            const T* row = pages + ((size_t)bt[p / page_size] * page_size + p % page_size) * DK;
+            const uint4 x = reinterpret_cast<const uint4*>(row)[v];
+            uint32_t* dst = tile + jj * row_words + 4 * v;
+            dst[0] = x.x; dst[1] = x.y; dst[2] = x.z; dst[3] = x.w;
+        }
+        __syncthreads();
+        float s0 = 0.f, s1 = 0.f;
+        if (j < cnt) {
+            const uint32_t* krow = tile + j * row_words;
+            const float* qa = qs + (2 * hp) * DK;
+            const float* qb = qa + DK;
+            for (int w = 0; w < words; ++w) {
+                float k[PER];
+                als_unpack<T>(krow[w], k);
+#pragma unroll
+                for (int u = 0; u < PER; ++u) {
+                    s0 = fmaf(qa[w * PER + u], k[u], s0);
+                    s1 = fmaf(qb[w * PER + u], k[u], s1);
+                }
+            }
+        } else {
+            s0 = s1 = -INFINITY;
+        }
+        // maximum and sum over the tile's keys: the 32 lanes that share a head pair are half a wave
+        float t0 = s0, t1 = s1;
+#pragma unroll
+        for (int o = ALS_TILE / 2; o > 0; o >>= 1) {
+            t0 = fmaxf(t0, __shfl_xor(t0, o, 64));
+            t1 = fmaxf(t1, __shfl_xor(t1, o, 64));
+        }
+        const float n0 = fmaxf(m0, t0), n1 = fmaxf(m1, t1);
+        const float p0 = j < cnt ? expf(s0 - n0) : 0.f, p1 = j < cnt ? expf(s1 - n1) : 0.f;
+        float u0 = p0, u1 = p1;
+#pragma unroll
+        for (int o = ALS_TILE / 2; o > 0; o >>= 1) {
+            u0 += __shfl_xor(u0, o, 64);
+            u1 += __shfl_xor(u1, o, 64);
+        }
+        const float c0 = expf(m0 - n0), c1 = expf(m1 - n1);           // first tile: exp(-inf) = 0
+        l0 = l0 * c0 + u0; l1 = l1 * c1 + u1;
+        m0 = n0; m1 = n1;
+        ps[j * ALS_HEADS + 2 * hp] = p0;
+        ps[j * ALS_HEADS + 2 * hp + 1] = p1;
+        if (j == 0) {
+            cs[2 * hp] = c0;
+            cs[2 * hp + 1] = c1;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const int d = tid + c * ALS_THREADS;
+            if (d < R) {
+#pragma unroll
+                for (int hh = 0; hh < ALS_HEADS; ++hh) acc[c][hh] *= cs[hh];
+                for (int jj = 0; jj < cnt; ++jj) {
+                    float kv[PER];
+                    als_unpack<T>(tile[jj * row_words + d / PER], kv);
+                    const float v = kv[d % PER];
+                    const float4* pr = reinterpret_cast<const float4*>(ps + jj * ALS_HEADS);
+#pragma unroll
+                    for (int g = 0; g < ALS_HEADS / 4; ++g) {
+                        const float4 pp = pr[g];
+                        acc[c][4 * g] = fmaf(pp.x, v, acc[c][4 * g]);
+                        acc[c][4 * g + 1] = fmaf(pp.y, v, acc[c][4 * g + 1]);
+                        acc[c][4 * g + 2] = fmaf(pp.z, v, acc[c][4 * g + 2]);
+                        acc[c][4 * g + 3] = fmaf(pp.w, v, acc[c][4 * g + 3]);
+                    }
+                }
+            }
+        }
+    }
+    // the run's results: [row][head][run][R] and [row][head][run][2]
+    if (j == 0) {
+        for (int u = 0; u < 2; ++u) {
+            const int hh = 2 * hp + u;
+            if (hh < nh) {
+                float* ml = part_ml + (((size_t)tok * H + h0 + hh) * max_splits + split) * 2;
+                ml[0] = u ? m1 : m0;
+                ml[1] = u ? l1 : l0;
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const int d = tid + c * ALS_THREADS;
+        if (d < R) {
+#pragma unroll
+            for (int hh = 0; hh < ALS_HEADS; ++hh)
+                if (hh < nh) part_o[(((size_t)tok * H + h0 + hh) * max_splits + split) * R + d] = acc[c][hh];
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+attention_latent_join_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ positions,
+                             const int* __restrict__ token_seq, int H, int R, int max_splits, float* __restrict__ out, long ldo) {
+    const int tok = blockIdx.x, head = blockIdx.y;
+    float* o = out + (size_t)tok * ldo + (size_t)head * R;
+    if (token_seq[tok] < 0) {
+        for (int d = threadIdx.x; d < R; d += 256) o[d] = 0.f;
+        return;
+    }
+    const int runs = positions[tok] / ALS_SPLIT + 1;
+    const float* ml = part_ml + ((size_t)tok * H + head) * max_splits * 2;
+    float m = -INFINITY;
+    for (int s = 0; s < runs; ++s) m = fmaxf(m, ml[2 * s]);
+    float l = 0.f;
+    for (int s = 0; s < runs; ++s) l += expf(ml[2 * s] - m) * ml[2 * s + 1];
+    const float inv = 1.f / l;
+    const float* po = part_o + ((size_t)tok * H + head) * max_splits * R;
+    for (int d = threadIdx.x; d < R; d += 256) {
+        float a = 0.f;
+        for (int s = 0; s < runs; ++s) a = fmaf(expf(ml[2 * s] - m), po[(size_t)s * R + d], a);
+        o[d] = a * inv;
+    }
+}
+
+// bytes of LDS the split kernel needs for these sizes, and the pitch of a key row in it (32-bit words, odd)
+static void als_layout(int R, int DR, int elem, int& row_words, size_t& lds) {
+    const int words = (R + DR) * elem / 4;
+    row_words = words | 1;
+    lds = (size_t)ALS_HEADS * (R + DR) * 4 + (size_t)ALS_TILE * row_words * 4 + (size_t)ALS_TILE * ALS_HEADS * 4 + ALS_HEADS * 4;
+}
+
+// floats of scratch for n rows whose contexts reach max_context positions: (weighted sums, maxima and sums)
+extern "C" long mv_attention_latent_split_workspace(int n, int H, int R, int max_context) {
+    const long runs = (max_context + ALS_SPLIT - 1) / ALS_SPLIT;
+    return (long)n * H * runs * (R + 2);
+}
+
+// returns 2 (nothing done) when the sizes are not served: the caller takes the general kernel
+extern "C" int mv_attention_latent_split(const float* q, long ldq, float* out, long ldo, const void* pages, const int* block_table,
+                                         int bt_width, int page_size, const int* positions, const int* token_seq, int n, int H,
+                                         int R, int DR, float scale, int max_context, float* work, long work_floats, int dtype,
+                                         hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && H > 0 && R > 0 && DR >= 0 && max_context > 0, "attention_latent_split: bad sizes n=%d H=%d R=%d DR=%d", n, H, R, DR);
+    const int elem = (int)mv_dtype_size(dtype);
+    int row_words = 0;
+    size_t lds = 0;
+    als_layout(R, DR, elem, row_words, lds);
+    if (((R + DR) * elem) % 16 != 0 || ((uintptr_t)pages % 16) != 0 || R > 2 * ALS_THREADS || lds > 64 * 1024) return 2;
+    MV_REQUIRE(page_size > 0 && bt_width > 0 && ldq >= (long)H * (R + DR) && ldo >= (long)H * R, "attention_latent_split: pitches too small");
+    MV_REQUIRE(q && out && pages && block_table && positions && token_seq && work, "attention_latent_split: missing operand");
+    const int runs = (max_context + ALS_SPLIT - 1) / ALS_SPLIT;
+    MV_REQUIRE(work_floats >= mv_attention_latent_split_workspace(n, H, R, max_context) && runs <= 65535,
+               "attention_latent_split: scratch of %ld floats is too small", work_floats);
+    if (n == 0) return 0;
+    float* part_o = work;
+    float* part_ml = work + (size_t)n * H * runs * R;
+    dim3 grid(n, (H + ALS_HEADS - 1) / ALS_HEADS, runs);
+    MV_DISPATCH_T(dtype, "attention_latent_split",
+                  hipLaunchKernelGGL(attention_latent_split_kernel<T>, grid, dim3(ALS_THREADS), lds, stream, q, ldq, (const T*)pages,
+                                     block_table, bt_width, page_size, positions, token_seq, H, R, DR, scale, row_words, runs,
+                                     part_o, part_ml));
+    if (mv_check_launch("attention_latent_split")) return 1;
+    hipLaunchKernelGGL(attention_latent_join_kernel, dim3(n, H), dim3(256), 0, stream, part_o, part_ml, positions, token_seq, H, R,
+                       runs, out, ldo);
+    return mv_check_launch("attention_latent_join");
 }

@@ -172,6 +172,11 @@ _OPTIONAL_SIGNATURES = {
     # q, ldq, out, ldo, pages, block_table, bt_width, page_size, positions, token_seq, n, H, R, DR, scale, dtype, stream
     "mv_attention_latent": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p,
                                     c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
+    "mv_attention_latent_split_workspace": (c_long, [c_int, c_int, c_int, c_int]),
+    # as mv_attention_latent up to scale, then max_context, work, work_floats, dtype, stream
+    "mv_attention_latent_split": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                                          c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_long, c_int,
+                                          c_void_p]),
     # logits, ld, n, E, correction, weight_dtype, groups, keep, top, sum_eps, dense, ids, weights, stream
     "mv_moe_route": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
                              c_void_p, c_void_p]),

@@ -206,6 +206,7 @@ class Ops:
         self._mid_retired: list = []
         self._tile_work: Optional[torch.Tensor] = None     # partial sums of the tiled product when it splits K
         self._sample_work: Optional[torch.Tensor] = None
+        self._latent_work: Optional[torch.Tensor] = None   # per-run results of the latent attention's single-token kernel
         self._attn_counters: Optional[torch.Tensor] = None
         # measurement: with a list here, every launch leaves (entry point, bytes it has to move,
         # floating-point operations) in it; the benchmark sets it for one eager step and prices the
@@ -767,11 +768,35 @@ class Ops:
         self._ints(n, positions=(positions, n), token_seq=(token_seq, n))
         kv_tokens = plan.kv_tokens if plan is not None else 0
         pairs = plan.attention_pairs if plan is not None else 0
+        if plan is not None and plan.decode_only and plan.max_context_len > 0 and self._attention_latent_split(
+                q, out, pages, block_table, page_size, positions, token_seq, n, heads, kv_rank, rot_dim, scale,
+                plan.max_context_len, kv_tokens):
+            return
         self._note("mv_attention_latent", self._size(q, out) + kv_tokens * dk * pages.element_size(),
                    2 * pairs * heads * (dk + kv_rank))
         self.lib.call("mv_attention_latent", q.data_ptr(), heads * dk, out.data_ptr(), heads * kv_rank, pages.data_ptr(),
                       block_table.data_ptr(), block_table.shape[1], page_size, positions.data_ptr(), token_seq.data_ptr(),
                       n, heads, kv_rank, rot_dim, float(scale), self.code, self._stream())
+
+    def _attention_latent_split(self, q, out, pages, block_table, page_size, positions, token_seq, n, heads, kv_rank, rot_dim,
+                                scale, max_context, kv_tokens) -> bool:
+        """Steps of single tokens: each row's keys dealt out to workgroups in runs of 256 positions, every workgroup
+        serving 16 heads from key rows staged in LDS; False when the sizes are not served (the general kernel runs)."""
+        need = int(self.lib.dll.mv_attention_latent_split_workspace(n, heads, kv_rank, max_context))
+        if self._latent_work is None or self._latent_work.numel() < need:
+            if torch.cuda.is_current_stream_capturing():
+                return False                                   # no allocation inside a capture
+            if self._latent_work is not None:
+                self._mid_retired.append(self._latent_work)    # captured graphs may hold its address
+            self._latent_work = torch.empty(max(need, 1 << 20), dtype=torch.float32, device=q.device)
+        dk = kv_rank + rot_dim
+        if not self.lib.offer("mv_attention_latent_split", q.data_ptr(), heads * dk, out.data_ptr(), heads * kv_rank,
+                              pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size, positions.data_ptr(),
+                              token_seq.data_ptr(), n, heads, kv_rank, rot_dim, float(scale), int(max_context),
+                              self._latent_work.data_ptr(), self._latent_work.numel(), self.code, self._stream()):
+            return False
+        self._note("mv_attention_latent_split", self._size(q, out) + kv_tokens * dk * pages.element_size(), 0)
+        return True
 
     # ------------------------------------------------------------------------------------
     # mixture of experts

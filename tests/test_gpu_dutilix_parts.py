@@ -442,6 +442,50 @@ def test_latent_attention_finds_a_far_key(dtype):
     assert float(out[0, 0, 3]) < 3.0
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H, R, dr", [(16, 64, 16), (5, 32, 8), (20, 128, 32), (1, 16, 0), (3, 24, 8)])
+def test_latent_attention_single_token_kernel(dtype, H, R, dr):
+    """Steps of single tokens take a kernel that deals a row's keys out in runs of 256 positions and joins them: rows
+    whose contexts end just inside, at and just behind a run's border, one position long, and 900 long, with a padding
+    row, against the general kernel and against the softmax written out."""
+    from minivllm_amd.engine.step import AttentionPlan
+    ops = ops_for(dtype)
+    page_size, n_pages = 16, 64
+    ctx = [255, 256, 257, 1, 900, 512]
+    g = torch.Generator().manual_seed(H)
+    pages = torch.randn(n_pages * len(ctx), page_size, R + dr, generator=g).to(dtype).to(DEV)
+    width = -(-max(ctx) // page_size)
+    bt = torch.full((len(ctx), width), -1, dtype=torch.int32)
+    perm = torch.randperm(n_pages * len(ctx), generator=g)
+    used = 0
+    for s, c in enumerate(ctx):
+        need = -(-c // page_size)
+        bt[s, :need] = perm[used:used + need].to(torch.int32)
+        used += need
+    bt = bt.to(DEV)
+    n = len(ctx) + 1
+    qa = (1.5 * torch.randn(n, H, R + dr, generator=g)).to(DEV)
+    pos = i32([c - 1 for c in ctx] + [0]); tsq = i32(list(range(len(ctx))) + [-1])
+    plan = AttentionPlan(decode_only=True, max_q_len=1, max_context_len=1024, n_seqs=len(ctx))
+    fast = torch.full((n, H, R), float("nan"), device=DEV)
+    slow = torch.full((n, H, R), float("nan"), device=DEV)
+    ops.ledger = []
+    ops.attention_latent(qa, fast, pages, bt, page_size, pos, tsq, H, R, dr, 0.2, plan=plan)
+    taken = [e[0] for e in ops.ledger]
+    ops.ledger = None
+    ops.attention_latent(qa, slow, pages, bt, page_size, pos, tsq, H, R, dr, 0.2)
+    torch.cuda.synchronize()
+    assert taken == ["mv_attention_latent_split"], taken
+    assert (fast[-1] == 0).all()
+    stored = pages.float().cpu().double()
+    for s, c in enumerate(ctx):
+        rows = torch.stack([stored[bt[s, p // page_size].item(), p % page_size] for p in range(c)])
+        for h in range(H):
+            w = torch.softmax(rows @ qa[s, h].double().cpu() * 0.2, 0)
+            close(fast[s, h], w @ rows[:, :R], 3e-5, f"context {c} head {h}")
+    close(fast[:-1], slow[:-1].double(), 3e-5, "against the general kernel")
+
+
 # ---------------------------------------------------------------------------------------
 # router and experts
 # ---------------------------------------------------------------------------------------
