@@ -325,13 +325,13 @@ extern "C" int mv_attention_latent(const float* q, long ldq, float* out, long ld
 
 // ---------------------------------------------------------------------------------------
 // Attention for steps of few rows (single decoded tokens): a row's keys are dealt out to workgroups in
-// runs of ALS_SPLIT positions (run s holds positions s * ALS_SPLIT ..., so the cutting depends on the
-// position alone), a workgroup serves up to ALS_HEADS heads of the row at once and brings each tile of
+// runs of `run` positions (run s holds positions s * run ..., so the cutting depends on the position and
+// the launch's run length alone), a workgroup serves up to ALS_HEADS heads of the row at once and brings each tile of
 // ALS_TILE key rows into LDS with 16-byte loads, where all its heads read them. It leaves per run the
 // running maximum, the sum of weights and the weighted sum of latents; a second kernel joins the runs
 // in their order. Requires (R + DR) * sizeof(T) to be a multiple of 16.
 // ---------------------------------------------------------------------------------------
-#define ALS_SPLIT 256
+#define ALS_MAX_VEC 8          // 16-byte pieces of a tile a thread brings in: key rows of up to 1,024 bytes
 #define ALS_TILE 32
 #define ALS_HEADS 16
 #define ALS_THREADS 256
@@ -354,8 +354,8 @@ template <typename T>
 __global__ void __launch_bounds__(ALS_THREADS)
 attention_latent_split_kernel(const float* __restrict__ q, long ldq, const T* __restrict__ pages, const int* __restrict__ block_table,
                               int bt_width, int page_size, const int* __restrict__ positions, const int* __restrict__ token_seq,
-                              int H, int R, int DR, float scale, int row_words, int max_splits, float* __restrict__ part_o,
-                              float* __restrict__ part_ml) {
+                              int H, int R, int DR, float scale, int row_words, int run, int max_splits,
+                              float* __restrict__ part_o, float* __restrict__ part_ml) {
     extern __shared__ __attribute__((aligned(16))) unsigned char als_lds[];
     constexpr int PER = AlsWord<T>::per;
     const int DK = R + DR;
@@ -368,9 +368,9 @@ attention_latent_split_kernel(const float* __restrict__ q, long ldq, const T* __
     const int seq = token_seq[tok];
     if (seq < 0) return;
     const int pos = positions[tok];
-    const int lo = split * ALS_SPLIT;
+    const int lo = split * run;
     if (lo > pos) return;
-    const int hi = min(pos, lo + ALS_SPLIT - 1);
+    const int hi = min(pos, lo + run - 1);
     const int nh = min(ALS_HEADS, H - h0);
     const int* bt = block_table + (size_t)seq * bt_width;
     for (int e = tid; e < ALS_HEADS * DK; e += ALS_THREADS) {
@@ -386,17 +386,34 @@ attention_latent_split_kernel(const float* __restrict__ q, long ldq, const T* __
 #pragma unroll
         for (int hh = 0; hh < ALS_HEADS; ++hh) acc[c][hh] = 0.f;
     const int vec_per_row = words / 4;                      // 16-byte pieces of a key row
+    // a tile comes from memory into registers while the tile before it is computed, and from there into LDS
+    uint4 held[ALS_MAX_VEC];
+    auto fetch = [&](int base) {
+        const int cnt = min(ALS_TILE, hi - base + 1);
+#pragma unroll
+        for (int x = 0; x < ALS_MAX_VEC; ++x) {
+            const int e = tid + x * ALS_THREADS;
+            if (e < cnt * vec_per_row) {
+                const int jj = e / vec_per_row, v = e % vec_per_row;
+                const int p = base + jj;
+                const T* row = pages + ((size_t)bt[p / page_size] * page_size + p % page_size) * DK;
+                held[x] = reinterpret_cast<const uint4*>(row)[v];
+            }
+        }
+    };
+    fetch(lo);
     for (int base = lo; base <= hi; base += ALS_TILE) {
         const int cnt = min(ALS_TILE, hi - base + 1);
         __syncthreads();                                    // the tile before has been read (and qs is written)
-        for (int e = tid; e < cnt * vec_per_row; e += ALS_THREADS) {
-            const int jj = e / vec_per_row, v = e % vec_per_row;
-            const int p = base + jj;
-            const T* row = pages + ((size_t)bt[p / page_size] * page_size + p % page_size) * DK;
-            const uint4 x = reinterpret_cast<const uint4*>(row)[v];
-            uint32_t* dst = tile + jj * row_words + 4 * v;
-            dst[0] = x.x; dst[1] = x.y; dst[2] = x.z; dst[3] = x.w;
+#pragma unroll
+        for (int x = 0; x < ALS_MAX_VEC; ++x) {
+            const int e = tid + x * ALS_THREADS;
+            if (e < cnt * vec_per_row) {
+                uint32_t* dst = tile + (e / vec_per_row) * row_words + 4 * (e % vec_per_row);
+                dst[0] = held[x].x; dst[1] = held[x].y; dst[2] = held[x].z; dst[3] = held[x].w;
+            }
         }
+        if (base + ALS_TILE <= hi) fetch(base + ALS_TILE);
         __syncthreads();
         float s0 = 0.f, s1 = 0.f;
         if (j < cnt) {
@@ -447,9 +464,8 @@ attention_latent_split_kernel(const float* __restrict__ q, long ldq, const T* __
 #pragma unroll
                 for (int hh = 0; hh < ALS_HEADS; ++hh) acc[c][hh] *= cs[hh];
                 for (int jj = 0; jj < cnt; ++jj) {
-                    float kv[PER];
-                    als_unpack<T>(tile[jj * row_words + d / PER], kv);
-                    const float v = kv[d % PER];
+                    const uint32_t word = tile[jj * row_words + d / PER];
+                    const float v = PER == 1 ? __uint_as_float(word) : __uint_as_float((d & 1) ? (word & 0xffff0000u) : (word << 16));
                     const float4* pr = reinterpret_cast<const float4*>(ps + jj * ALS_HEADS);
 #pragma unroll
                     for (int g = 0; g < ALS_HEADS / 4; ++g) {
@@ -487,14 +503,15 @@ attention_latent_split_kernel(const float* __restrict__ q, long ldq, const T* __
 
 __global__ void __launch_bounds__(256)
 attention_latent_join_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ positions,
-                             const int* __restrict__ token_seq, int H, int R, int max_splits, float* __restrict__ out, long ldo) {
+                             const int* __restrict__ token_seq, int H, int R, int run, int max_splits, float* __restrict__ out,
+                             long ldo) {
     const int tok = blockIdx.x, head = blockIdx.y;
     float* o = out + (size_t)tok * ldo + (size_t)head * R;
     if (token_seq[tok] < 0) {
         for (int d = threadIdx.x; d < R; d += 256) o[d] = 0.f;
         return;
     }
-    const int runs = positions[tok] / ALS_SPLIT + 1;
+    const int runs = positions[tok] / run + 1;
     const float* ml = part_ml + ((size_t)tok * H + head) * max_splits * 2;
     float m = -INFINITY;
     for (int s = 0; s < runs; ++s) m = fmaxf(m, ml[2 * s]);
@@ -516,9 +533,14 @@ static void als_layout(int R, int DR, int elem, int& row_words, size_t& lds) {
     lds = (size_t)ALS_HEADS * (R + DR) * 4 + (size_t)ALS_TILE * row_words * 4 + (size_t)ALS_TILE * ALS_HEADS * 4 + ALS_HEADS * 4;
 }
 
+// positions of a run: short runs while that keeps their number small (a workgroup's tiles follow one another,
+// so few tiles a workgroup and many workgroups is what a step of few rows wants)
+static int als_run(int max_context) { return max_context <= 8192 ? 64 : (max_context <= 32768 ? 256 : 1024); }
+
 // floats of scratch for n rows whose contexts reach max_context positions: (weighted sums, maxima and sums)
 extern "C" long mv_attention_latent_split_workspace(int n, int H, int R, int max_context) {
-    const long runs = (max_context + ALS_SPLIT - 1) / ALS_SPLIT;
+    const int run = als_run(max_context);
+    const long runs = (max_context + run - 1) / run;
     return (long)n * H * runs * (R + 2);
 }
 
@@ -532,10 +554,12 @@ extern "C" int mv_attention_latent_split(const float* q, long ldq, float* out, l
     int row_words = 0;
     size_t lds = 0;
     als_layout(R, DR, elem, row_words, lds);
-    if (((R + DR) * elem) % 16 != 0 || ((uintptr_t)pages % 16) != 0 || R > 2 * ALS_THREADS || lds > 64 * 1024) return 2;
+    if (((R + DR) * elem) % 16 != 0 || ((uintptr_t)pages % 16) != 0 || R > 2 * ALS_THREADS || lds > 64 * 1024
+        || ALS_TILE * ((R + DR) * elem / 16) > ALS_MAX_VEC * ALS_THREADS) return 2;
     MV_REQUIRE(page_size > 0 && bt_width > 0 && ldq >= (long)H * (R + DR) && ldo >= (long)H * R, "attention_latent_split: pitches too small");
     MV_REQUIRE(q && out && pages && block_table && positions && token_seq && work, "attention_latent_split: missing operand");
-    const int runs = (max_context + ALS_SPLIT - 1) / ALS_SPLIT;
+    const int run = als_run(max_context);
+    const int runs = (max_context + run - 1) / run;
     MV_REQUIRE(work_floats >= mv_attention_latent_split_workspace(n, H, R, max_context) && runs <= 65535,
                "attention_latent_split: scratch of %ld floats is too small", work_floats);
     if (n == 0) return 0;
@@ -544,10 +568,10 @@ extern "C" int mv_attention_latent_split(const float* q, long ldq, float* out, l
     dim3 grid(n, (H + ALS_HEADS - 1) / ALS_HEADS, runs);
     MV_DISPATCH_T(dtype, "attention_latent_split",
                   hipLaunchKernelGGL(attention_latent_split_kernel<T>, grid, dim3(ALS_THREADS), lds, stream, q, ldq, (const T*)pages,
-                                     block_table, bt_width, page_size, positions, token_seq, H, R, DR, scale, row_words, runs,
+                                     block_table, bt_width, page_size, positions, token_seq, H, R, DR, scale, row_words, run, runs,
                                      part_o, part_ml));
     if (mv_check_launch("attention_latent_split")) return 1;
     hipLaunchKernelGGL(attention_latent_join_kernel, dim3(n, H), dim3(256), 0, stream, part_o, part_ml, positions, token_seq, H, R,
-                       runs, out, ldo);
+                       run, runs, out, ldo);
     return mv_check_launch("attention_latent_join");
 }
