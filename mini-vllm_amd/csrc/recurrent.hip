@@ -796,7 +796,7 @@ mlstm_gates_kernel(const T* __restrict__ packed, long ld, int H, long gate_off, 
         const int t = base + lane;
         const bool live = t < end;
         const T* p = packed + (size_t)(live ? t : first) * ld + gate_off;
-        const float gi = cap * tanhf((to_f(p[head]) + bi) / cap);
+        const float gi = __fmul_rn(cap, tanhf((to_f(p[head]) + bi) / cap));      // (rounded here: never fused into a later sum)
         const float gf = logsigmoid_f(cap * tanhf((to_f(p[H + head]) + bf) / cap));
         // the maximum runs token by token, in the same order however the request was cut into steps: every lane
         // walks the 64 rows (their gates come by lane broadcasts), lane j keeps the values of row j
@@ -869,6 +869,26 @@ extern "C" int mv_mlstm_prepare(const void* packed, long ld, int n, int n_seqs, 
 // above). The vectors of a run of tokens are staged in LDS; the additions of a token depend on
 // nothing but the sizes, so a token computed alone has the bits it has inside a prompt.
 // ---------------------------------------------------------------------------------------
+// one token of one column: the lane's R rows of the column in s, its R channels of q and k; returns the column's output
+template <int R, int L, bool READ>
+__device__ __forceinline__ float state_update(float (&s)[R], const float (&q)[R], const float (&k)[R], float a, float b, float v) {
+    float u = v;
+    if constexpr (READ) {
+        float read = 0.f;
+#pragma unroll
+        for (int e = 0; e < R; ++e) read = fmaf(k[e], s[e], read);
+        u = v - a * lanes_sum<L>(read);
+    }
+    u *= b;
+    float o = 0.f;
+#pragma unroll
+    for (int e = 0; e < R; ++e) {
+        s[e] = fmaf(a, s[e], k[e] * u);
+        o = fmaf(q[e], s[e], o);
+    }
+    return lanes_sum<L>(o);
+}
+
 template <int R, int L, bool READ>
 __global__ void __launch_bounds__(256)
 state_scan_kernel(const float* __restrict__ qk, const float* __restrict__ vals, const float* __restrict__ gates,
@@ -911,21 +931,7 @@ state_scan_kernel(const float* __restrict__ qk, const float* __restrict__ vals, 
                 q[e] = sv[tt][0][sub * R + e];
                 k[e] = sv[tt][1][sub * R + e];
             }
-            float u = v;
-            if constexpr (READ) {
-                float read = 0.f;
-#pragma unroll
-                for (int e = 0; e < R; ++e) read = fmaf(k[e], s[e], read);
-                u = v - a * lanes_sum<L>(read);
-            }
-            u *= b;
-            float o = 0.f;
-#pragma unroll
-            for (int e = 0; e < R; ++e) {
-                s[e] = fmaf(a, s[e], k[e] * u);
-                o = fmaf(q[e], s[e], o);
-            }
-            o = lanes_sum<L>(o);
+            const float o = state_update<R, L, READ>(s, q, k, a, b, v);
             if (live && sub == 0) out[((size_t)(base + tt) * H + head) * DV + j] = o;
         }
     }
@@ -1020,4 +1026,211 @@ extern "C" int mv_state_finish(const float* raw, const float* gates, const void*
                                      (const T*)packed, ld, g_off, w, shared_weight, silu_gate, normaliser, denom_eps, H, DV,
                                      DV + (normaliser ? 1 : 0), eps, token_seq, (T*)out, ldo, n));
     return mv_check_launch("state_finish");
+}
+
+// ---------------------------------------------------------------------------------------
+// A step of single tokens: prepare, the recurrence and finish of one (row, head) in one workgroup, for both
+// mixers (READ: the gated delta rule, whose convolution reads the request's kept inputs; they are advanced by
+// conv_state_kernel afterwards, since the heads of a group share them. Otherwise the mLSTM, whose running
+// maximum belongs to the head and is advanced here). Sums run in the order of the kernels above, so a token
+// computed here has the bits it has as a prompt's last token.
+// ---------------------------------------------------------------------------------------
+struct StepArgs {
+    const void* packed; long ld;
+    int H, G, DK, DV, taps;
+    WeightPtr conv_w, a_log, dt_bias, i_bias, f_bias, norm_w;
+    const void* conv_state; float* max_state; float* state;
+    float unit_eps, cap, denom_eps, eps;
+    const int* token_seq; const int* state_slots;
+    void* out; long ldo;
+};
+
+template <typename T, int R, int L, bool READ>
+__global__ void __launch_bounds__(256)
+state_step_kernel(StepArgs A) {
+    constexpr int DPAD = L * R;
+    constexpr int COLS = 256 / L;
+    __shared__ float vq[DPAD], vk[DPAD];
+    __shared__ float vals[260], outs[260];
+    __shared__ float red[8];
+    const int H = A.H, G = A.G, DK = A.DK, DV = A.DV;
+    const int DVS = READ ? DV : DV + 1;                     // columns of the state
+    const int t = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+    const int lane = tid % MV_WAVE, wave = tid / MV_WAVE;
+    const int seq = A.token_seq[t];
+    T* y = (T*)A.out + (size_t)t * A.ldo + (size_t)head * DV;
+    if (seq < 0) {
+        for (int d = tid; d < DV; d += 256) y[d] = from_f<T>(0.f);
+        return;
+    }
+    const int slot = A.state_slots[seq];
+    const T* packed = (const T*)A.packed;
+    const T* p = packed + (size_t)t * A.ld;
+    long g_off;
+    if constexpr (READ) {
+        const int C = 2 * G * DK + H * DV, taps = A.taps;
+        const int group = head / (H / G);
+        const T* hist = (const T*)A.conv_state + (size_t)slot * (taps - 1) * C;
+        // the row is its request's only one in the step: every earlier input comes from the kept ones
+        auto conv = [&](int c) {
+            float acc = 0.f;
+            for (int j = 0; j < taps - 1; ++j) acc = fmaf(A.conv_w.at((size_t)c * taps + j), to_f(hist[(size_t)j * C + c]), acc);
+            acc = fmaf(A.conv_w.at((size_t)c * taps + taps - 1), to_f(p[c]), acc);
+            return silu_f(acc);
+        };
+        // as the prepare kernel sums: 128 threads over the channels, a wave's sum, the waves in order
+        float sq = 0.f, sk = 0.f, xq[2] = {0.f, 0.f}, xk[2] = {0.f, 0.f};
+        if (tid < 128) {
+            int u = 0;
+            for (int d = tid; d < DK; d += 128, ++u) {
+                xq[u] = conv(group * DK + d);
+                xk[u] = conv(G * DK + group * DK + d);
+                sq = fmaf(xq[u], xq[u], sq);
+                sk = fmaf(xk[u], xk[u], sk);
+            }
+            sq = wave_sum(sq);
+            sk = wave_sum(sk);
+            if (lane == 0) {
+                red[wave] = sq;
+                red[2 + wave] = sk;
+            }
+        }
+        for (int d = tid; d < DV; d += 256) vals[d] = conv(2 * G * DK + head * DV + d);
+        __syncthreads();
+        if (tid < 128) {
+            const float iq = (1.f / sqrtf((float)DK)) / sqrtf((0.f + red[0]) + red[1] + A.unit_eps);
+            const float ik = 1.f / sqrtf((0.f + red[2]) + red[3] + A.unit_eps);
+            int u = 0;
+            for (int d = tid; d < DPAD; d += 128, ++u) {
+                vq[d] = d < DK ? xq[u] * iq : 0.f;
+                vk[d] = d < DK ? xk[u] * ik : 0.f;
+            }
+        }
+        if (tid == 0) {
+            const T* gp = p + C + (size_t)H * DV;
+            red[4] = expf(-expf(A.a_log.at(head)) * softplus_f(to_f(gp[H + head]) + A.dt_bias.at(head)));
+            red[5] = sigmoid_f(to_f(gp[head]));
+            red[6] = 0.f;
+        }
+        g_off = C;
+    } else {
+        const float qs = 1.f / sqrtf((float)DK);
+        for (int d = tid; d < DPAD; d += 256) {
+            vq[d] = d < DK ? to_f(p[(size_t)head * DK + d]) * qs : 0.f;
+            vk[d] = d < DK ? to_f(p[(size_t)(H + head) * DK + d]) : 0.f;
+        }
+        for (int d = tid; d < DV; d += 256) vals[d] = to_f(p[2 * (size_t)H * DK + (size_t)head * DV + d]);
+        g_off = 2L * H * DK + (long)H * DV;
+        if (tid == 0) {
+            vals[DV] = 1.f;
+            const T* gp = p + g_off + (size_t)H * DV;
+            const float gi = __fmul_rn(A.cap, tanhf((to_f(gp[head]) + A.i_bias.at(head)) / A.cap));
+            const float gf = logsigmoid_f(A.cap * tanhf((to_f(gp[H + head]) + A.f_bias.at(head)) / A.cap));
+            float* ms = A.max_state + (size_t)slot * H + head;
+            const float m = *ms;
+            const float m_new = fmaxf(gf + m, gi);
+            red[4] = expf(gf + m - m_new);
+            red[5] = expf(gi - m_new);
+            red[6] = expf(-m_new);
+            *ms = m_new;
+        }
+    }
+    __syncthreads();
+    const float a = red[4], b = red[5];
+    const int sub = tid % L, col = tid / L;
+    float q[R], k[R];
+#pragma unroll
+    for (int e = 0; e < R; ++e) {
+        q[e] = vq[sub * R + e];
+        k[e] = vk[sub * R + e];
+    }
+    float* S0 = A.state + ((size_t)slot * H + head) * (size_t)DVS * DK;
+    float s[R], s_next[R];
+    delta_state_io<R, false>(s, S0 + (size_t)(col < DVS ? col : 0) * DK, sub, DK, col < DVS);
+    for (int j0 = 0; j0 < DVS; j0 += COLS) {
+        const int j = j0 + col;
+        const bool live = j < DVS;
+        const int jn = j + COLS;
+        if (j0 + COLS < DVS) delta_state_io<R, false>(s_next, S0 + (size_t)(jn < DVS ? jn : 0) * DK, sub, DK, jn < DVS);
+        const float o = state_update<R, L, READ>(s, q, k, a, b, vals[live ? j : 0]);
+        delta_state_io<R, true>(s, S0 + (size_t)(live ? j : 0) * DK, sub, DK, live);
+        if (live && sub == 0) outs[j] = o;
+#pragma unroll
+        for (int e = 0; e < R; ++e) s[e] = s_next[e];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float scale = 1.f;
+        if constexpr (!READ) scale = 1.f / (fmaxf(fabsf(outs[DV]), red[6]) + A.denom_eps);
+        float ss = 0.f;
+        for (int d = lane; d < DV; d += MV_WAVE) {
+            const float x = outs[d] * scale;
+            ss = fmaf(x, x, ss);
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) red[7] = scale / sqrtf(ss / (float)DV + A.eps);
+    }
+    __syncthreads();
+    const float rinv = red[7];
+    const T* g = p + g_off + (size_t)head * DV;
+    for (int d = tid; d < DV; d += 256) {
+        const float z = to_f(g[d]);
+        const float act = READ ? silu_f(z) : sigmoid_f(z);
+        y[d] = from_f<T>(outs[d] * rinv * A.norm_w.at(READ ? d : (size_t)head * DV + d) * act);
+    }
+}
+
+// mode 1: gated delta rule (conv_state, conv_w, a_log, dt_bias); mode 0: mLSTM (max_state, i_bias, f_bias, cap).
+// Returns 2 (nothing done) for sizes it does not serve.
+extern "C" int mv_state_step(int mode, const void* packed, long ld, int n, int n_seqs, int H, int G, int DK, int DV, int taps,
+                             const void* conv_w, const void* a_log, const void* dt_bias, const void* i_bias,
+                             const void* f_bias, const void* norm_w, int weight_dtype, void* conv_state, float* max_state,
+                             float* state, float unit_eps, float cap, float denom_eps, float eps, const int* token_seq,
+                             const int* cu_seqlens, const int* state_slots, void* out, long ldo, int dtype,
+                             hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0 && DK > 0 && DV > 0, "state_step: bad sizes n=%d H=%d G=%d DK=%d DV=%d", n, H, G, DK, DV);
+    if (DK > 256 || DV + 1 > 260 || (mode == 1 && (taps < 1 || taps > MS_MAX_TAPS))) return 2;
+    MV_REQUIRE(mv_valid_dtype(weight_dtype) && packed && norm_w && state && token_seq && cu_seqlens && state_slots && out,
+               "state_step: missing operand");
+    MV_REQUIRE(mode == 1 ? (conv_w && a_log && dt_bias && (conv_state || taps == 1) && unit_eps > 0.f)
+                         : (i_bias && f_bias && max_state && cap > 0.f), "state_step: missing operand of the mode");
+    MV_REQUIRE(eps > 0.f && H <= 65535 && ldo >= (long)H * DV, "state_step: bad constants");
+    if (n == 0) return 0;
+    StepArgs A;
+    A.packed = packed; A.ld = ld; A.H = H; A.G = G; A.DK = DK; A.DV = DV; A.taps = taps;
+    A.conv_w = WeightPtr{conv_w, weight_dtype}; A.a_log = WeightPtr{a_log, weight_dtype}; A.dt_bias = WeightPtr{dt_bias, weight_dtype};
+    A.i_bias = WeightPtr{i_bias, weight_dtype}; A.f_bias = WeightPtr{f_bias, weight_dtype}; A.norm_w = WeightPtr{norm_w, weight_dtype};
+    A.conv_state = conv_state; A.max_state = max_state; A.state = state;
+    A.unit_eps = unit_eps; A.cap = cap; A.denom_eps = denom_eps; A.eps = eps;
+    A.token_seq = token_seq; A.state_slots = state_slots; A.out = out; A.ldo = ldo;
+    int R = 0, L = 0;
+    delta_scan_shape(DK, R, L);
+    dim3 grid(n, H);
+#define SS_LAUNCH(RR, LL)                                                                                              \
+    if (mode == 1) {                                                                                                   \
+        MV_DISPATCH_T(dtype, "state_step", hipLaunchKernelGGL((state_step_kernel<T, RR, LL, true>), grid, dim3(256), 0, stream, A)) \
+    } else {                                                                                                           \
+        MV_DISPATCH_T(dtype, "state_step", hipLaunchKernelGGL((state_step_kernel<T, RR, LL, false>), grid, dim3(256), 0, stream, A)) \
+    }
+    if (R == 4 && L == 4) {
+        SS_LAUNCH(4, 4)
+    } else if (R == 4 && L == 8) {
+        SS_LAUNCH(4, 8)
+    } else if (R == 4 && L == 16) {
+        SS_LAUNCH(4, 16)
+    } else if (R == 8 && L == 16) {
+        SS_LAUNCH(8, 16)
+    } else {
+        SS_LAUNCH(16, 16)
+    }
+#undef SS_LAUNCH
+    if (mv_check_launch("state_step")) return 1;
+    if (mode == 1 && taps > 1 && n_seqs > 0) {
+        const long C = 2L * G * DK + (long)H * DV;
+        MV_DISPATCH_T(dtype, "conv_state",
+                      hipLaunchKernelGGL(conv_state_kernel<T>, dim3(n_seqs, (unsigned)((C + 255) / 256)), dim3(256), 0, stream,
+                                         (const T*)packed, ld, (int)C, taps, (T*)conv_state, cu_seqlens, state_slots));
+        return mv_check_launch("conv_state");
+    }
+    return 0;
 }

@@ -156,6 +156,11 @@ _OPTIONAL_SIGNATURES = {
     # qk, vals, gates, state, cu_seqlens, state_slots, n_seqs, n, H, G, DK, DV, read, out, stream
     "mv_state_scan": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                               c_int, c_int, c_void_p, c_void_p]),
+    # mode, packed, ld, n, n_seqs, H, G, DK, DV, taps, conv_w, a_log, dt_bias, i_bias, f_bias, norm_w, weight_dtype, conv_state,
+    # max_state, state, unit_eps, cap, denom_eps, eps, token_seq, cu_seqlens, state_slots, out, ldo, dtype, stream
+    "mv_state_step": (c_int, [c_int, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                              c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float, c_float,
+                              c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_int, c_void_p]),
     # raw, gates, packed, ld, g_off, weight, weight_dtype, shared_weight, silu_gate, normaliser, denom_eps, n, H, DV, eps,
     # token_seq, out, ldo, dtype, stream
     "mv_state_finish": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_long, c_void_p, c_int, c_int, c_int, c_int, c_float,

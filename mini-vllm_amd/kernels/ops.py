@@ -670,6 +670,57 @@ class Ops:
                       float(denom_eps), n, heads, dv, float(eps), token_seq.data_ptr(), out.data_ptr(),
                       out.stride(0) if n > 1 else heads * dv, self.code, self._stream())
 
+    def state_step(self, delta: bool, packed: torch.Tensor, heads: int, groups: int, dk: int, dv: int, norm_weight: torch.Tensor,
+                   eps: float, state: torch.Tensor, token_seq: torch.Tensor, cu_seqlens: torch.Tensor, state_slots: torch.Tensor,
+                   n_seqs: int, out: torch.Tensor, taps: int = 1, conv_w: Optional[torch.Tensor] = None,
+                   a_log: Optional[torch.Tensor] = None, dt_bias: Optional[torch.Tensor] = None,
+                   conv_state: Optional[torch.Tensor] = None, unit_eps: float = 1e-6, i_bias: Optional[torch.Tensor] = None,
+                   f_bias: Optional[torch.Tensor] = None, cap: float = 1.0, max_state: Optional[torch.Tensor] = None,
+                   denom_eps: float = 0.0) -> bool:
+        """For a step in which every request brings one token: the prepare kernel, ``state_scan`` and ``state_finish`` of
+        the gated delta rule (``delta``) or of the mLSTM as one kernel per (row, head), with the same sums in the same
+        order. False when the sizes are not served (nothing was done)."""
+        self._act(packed, "mixer rows"); self._act(out, "mixer output"); _dev(norm_weight, "output norm weight")
+        n = packed.shape[0]
+        dvs = dv if delta else dv + 1
+        width = (2 * groups * dk + 2 * heads * dv + 2 * heads) if delta else (2 * heads * (dk + dv) + 2 * heads)
+        if packed.dim() != 2 or packed.stride(1) != 1 or packed.shape[1] < width or tuple(out.shape) != (n, heads * dv) \
+                or out.stride(1) != 1 or norm_weight.numel() != (dv if delta else heads * dv) or not norm_weight.is_contiguous():
+            raise KernelLibraryError("state_step: operands do not fit")
+        _dev(state, "matrix state")
+        if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dvs, dk) or not state.is_contiguous():
+            raise KernelLibraryError(f"state_step: the state must be float32 [slots, {heads}, {dvs}, {dk}]")
+        wcode = _weight_code(norm_weight, "output norm weight")
+        if delta:
+            C = 2 * groups * dk + heads * dv
+            for t, shape, name in ((conv_w, (C, taps), "convolution taps"), (a_log, (heads,), "A_log"), (dt_bias, (heads,), "dt_bias")):
+                _dev(t, name)
+                if tuple(t.shape) != shape or not t.is_contiguous() or t.dtype != norm_weight.dtype:
+                    raise KernelLibraryError(f"state_step: {name} must be a contiguous {shape} tensor of the norm weight's dtype")
+            if taps > 1:
+                self._act(conv_state, "convolution state")
+                if conv_state.dim() != 3 or tuple(conv_state.shape[1:]) != (taps - 1, C) or not conv_state.is_contiguous():
+                    raise KernelLibraryError(f"state_step: the convolution's state must be [slots, {taps - 1}, {C}]")
+        else:
+            for t, name in ((i_bias, "input gate bias"), (f_bias, "forget gate bias")):
+                _dev(t, name)
+                if t.numel() != heads or not t.is_contiguous() or t.dtype != norm_weight.dtype:
+                    raise KernelLibraryError(f"state_step: the {name} must hold {heads} numbers of the norm weight's dtype")
+            _dev(max_state, "running maximum")
+            if max_state.dtype != torch.float32 or max_state.dim() != 2 or max_state.shape[1] != heads or not max_state.is_contiguous():
+                raise KernelLibraryError(f"state_step: the running maximum must be float32 [slots, {heads}]")
+        self._ints(n, token_seq=(token_seq, n), cu_seqlens=(cu_seqlens, n_seqs + 1), state_slots=(state_slots, n_seqs))
+        if not self.lib.offer("mv_state_step", int(bool(delta)), packed.data_ptr(), packed.stride(0) if n > 1 else packed.shape[1],
+                              n, n_seqs, heads, groups, dk, dv, taps, _ptr(conv_w), _ptr(a_log), _ptr(dt_bias), _ptr(i_bias),
+                              _ptr(f_bias), norm_weight.data_ptr(), wcode, _ptr(conv_state), _ptr(max_state), state.data_ptr(),
+                              float(unit_eps), float(cap), float(denom_eps), float(eps), token_seq.data_ptr(),
+                              cu_seqlens.data_ptr(), state_slots.data_ptr(), out.data_ptr(),
+                              out.stride(0) if n > 1 else heads * dv, self.code, self._stream()):
+            return False
+        self._note("mv_state_step", n * width * packed.element_size() + self._size(out) + 2 * n * heads * dvs * dk * 4,
+                   (6 if delta else 4) * n * heads * dvs * dk)
+        return True
+
     # ------------------------------------------------------------------------------------
     # attention over a cached latent
     def latent_prepare(self, packed: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, q_norm: torch.Tensor,

@@ -103,13 +103,23 @@ class GatedDelta(Mixer):
         self.conv_w = torch.cat([tensors["q_conv"], tensors["k_conv"], tensors["v_conv"]], dim=0).contiguous()
         self.a_log = tensors["A_log"].to(self.conv_w.dtype).contiguous()
         self.dt_bias = tensors["dt_bias"].to(self.conv_w.dtype).contiguous()
-        self.norm, self.w_o = tensors["norm"], tensors["o"]
+        self.norm, self.w_o = tensors["norm"].to(self.conv_w.dtype).contiguous(), tensors["o"]
 
     def forward(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
         spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
         n, H, G, dk, dv = x.shape[0], spec.num_heads, spec.num_kv_heads, spec.key_dim, spec.value_dim
         packed = ws.get("mstate.packed", (n, self.width), rt.dtype)
         ops.gemm(x, self.w_packed, packed)
+        gated = ws.get("mstate.gated", (n, H * dv), rt.dtype)
+        y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
+        plan = ctx.attention_plan
+        # every request brings one token: everything between the two products as one kernel
+        if plan is not None and plan.decode_only and ops.state_step(
+                True, packed, H, G, dk, dv, self.norm, spec.out_norm_eps, ctx.state(call), ctx.token_seq, ctx.cu_seqlens,
+                ctx.state_slots, ctx.n_seqs, gated, taps=spec.conv_taps, conv_w=self.conv_w, a_log=self.a_log,
+                dt_bias=self.dt_bias, conv_state=ctx.state(call, "conv") if spec.conv_taps > 1 else None,
+                unit_eps=spec.unit_eps):
+            return ops.gemm(gated, self.w_o, y, defer_sum=True) or y
         qk = ws.get("mstate.qk", (n, G, 2, dk), torch.float32)
         vals = ws.get("mstate.vals", (n, H, dv), torch.float32)
         gates = ws.get("mstate.gates", (n, H, 4), torch.float32)
@@ -118,10 +128,8 @@ class GatedDelta(Mixer):
                                 ctx.cu_seqlens, ctx.state_slots, ctx.n_seqs, qk, vals, gates)
         raw = ws.get("mstate.raw", (n, H, dv), torch.float32)
         ops.state_scan(qk, vals, gates, ctx.state(call), ctx.cu_seqlens, ctx.state_slots, ctx.n_seqs, H, G, dk, dv, True, raw)
-        gated = ws.get("mstate.gated", (n, H * dv), rt.dtype)
         ops.state_finish(raw, gates, packed, self.gate_offset, self.norm, H, dv, spec.out_norm_eps, ctx.token_seq, gated,
                          shared_weight=True, silu_gate=True)
-        y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
         return ops.gemm(gated, self.w_o, y, defer_sum=True) or y
 
 
@@ -166,13 +174,21 @@ class MLSTM(Mixer):
         self.gate_offset = spec.num_heads * (2 * spec.key_dim + spec.value_dim)
         self.i_bias = tensors["i_bias"].contiguous()
         self.f_bias = tensors["f_bias"].to(self.i_bias.dtype).contiguous()
-        self.norm, self.w_o = tensors["norm"], tensors["o"]
+        self.norm, self.w_o = tensors["norm"].to(self.i_bias.dtype).contiguous(), tensors["o"]
 
     def forward(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
         spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
         n, H, dk, dv = x.shape[0], spec.num_heads, spec.key_dim, spec.value_dim
         packed = ws.get("mstate.packed", (n, self.width), rt.dtype)
         ops.gemm(x, self.w_packed, packed)
+        gated = ws.get("mstate.gated", (n, H * dv), rt.dtype)
+        y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
+        plan = ctx.attention_plan
+        if plan is not None and plan.decode_only and ops.state_step(
+                False, packed, H, H, dk, dv, self.norm, spec.out_norm_eps, ctx.state(call), ctx.token_seq, ctx.cu_seqlens,
+                ctx.state_slots, ctx.n_seqs, gated, i_bias=self.i_bias, f_bias=self.f_bias, cap=spec.gate_cap,
+                max_state=ctx.state(call, "max"), denom_eps=spec.denom_eps):
+            return ops.gemm(gated, self.w_o, y, defer_sum=True) or y
         qk = ws.get("mstate.qk", (n, H, 2, dk), torch.float32)
         vals = ws.get("mstate.vals", (n, H, dv + 1), torch.float32)
         gates = ws.get("mstate.gates", (n, H, 4), torch.float32)
@@ -180,8 +196,6 @@ class MLSTM(Mixer):
                           ctx.cu_seqlens, ctx.state_slots, ctx.n_seqs, qk, vals, gates)
         raw = ws.get("mstate.raw", (n, H, dv + 1), torch.float32)
         ops.state_scan(qk, vals, gates, ctx.state(call), ctx.cu_seqlens, ctx.state_slots, ctx.n_seqs, H, H, dk, dv + 1, False, raw)
-        gated = ws.get("mstate.gated", (n, H * dv), rt.dtype)
         ops.state_finish(raw, gates, packed, self.gate_offset, self.norm, H, dv, spec.out_norm_eps, ctx.token_seq, gated,
                          shared_weight=False, silu_gate=False, normaliser=True, denom_eps=spec.denom_eps)
-        y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
         return ops.gemm(gated, self.w_o, y, defer_sum=True) or y

@@ -177,6 +177,43 @@ def test_a_written_value_is_read_back_and_decays():
     assert torch.allclose(raw[5, 0].cpu(), vals[4, 0].cpu() * 0.5)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H, G, dk, dv, taps", DELTA_SIZES)
+def test_gated_delta_single_token_kernel(dtype, H, G, dk, dv, taps):
+    """Steps of single tokens take one kernel per (row, head) instead of three: three such steps of four requests on
+    slots out of order, a padding row and a padding sequence, give the bits of the three kernels, states and kept
+    inputs included."""
+    ops = ops_for(dtype)
+    eps, slots, steps = 1e-5, [2, 0, 3, 1], 3
+    n = len(slots) + 1
+    C = 2 * G * dk + H * dv
+    g = torch.Generator().manual_seed(5)
+    S0 = 0.3 * torch.randn(5, H, dv, dk, generator=g)
+    hist0 = torch.randn(5, max(taps - 1, 1), C, generator=g).to(dtype)
+    results = []
+    for fused in (False, True):
+        state = S0.to(DEV).clone()
+        conv_state = hist0.to(DEV).clone() if taps > 1 else None
+        outs = []
+        for step in range(steps):
+            packed, t = delta_setup(H, G, dk, dv, taps, n, seed=50 + step, dtype=dtype)
+            if not fused:
+                outs.append(run_delta(ops, packed, t, H, G, dk, dv, taps, eps, conv_state, state, [1] * 4, slots, pad_rows=1, pad_seqs=1)[1].clone())
+                continue
+            tsq, cu, sl = step_ints([1] * 4, slots, 1, 1)
+            dev = {k: v.to(DEV) for k, v in t.items()}
+            out = torch.full((n, H * dv), 5.0, dtype=dtype, device=DEV)
+            assert ops.state_step(True, packed.to(DEV), H, G, dk, dv, dev["norm"], eps, state, tsq, cu, sl, 5, out, taps=taps,
+                                  conv_w=dev["conv"], a_log=dev["a_log"], dt_bias=dev["dt_bias"], conv_state=conv_state,
+                                  unit_eps=plain.UNIT_EPS)
+            torch.cuda.synchronize()
+            outs.append(out.clone())
+        results.append((torch.cat(outs), state.clone(), None if conv_state is None else conv_state.clone()))
+    assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+    assert taps == 1 or torch.equal(results[0][2], results[1][2])
+    assert torch.equal(results[1][1][4].cpu(), S0[4])
+
+
 # ---------------------------------------------------------------------------------------
 # mLSTM
 # ---------------------------------------------------------------------------------------
@@ -284,6 +321,39 @@ def test_mlstm_one_by_one_against_the_prompt(dtype):
         outs.append(torch.cat(rows))
     assert torch.equal(outs[1], outs[0]), "one by one against whole"
     close(outs[1], mlstm_plain(packed, t, H, dk, dv, cap, eps, [None] * H)[1], 3e-5 if dtype == torch.float32 else 1.2e-2, "plain")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H, dk, dv, cap", [(2, 16, 20, 10.0), (3, 10, 6, 15.0), (2, 128, 64, 12.0), (1, 8, 12, 4.0), (4, 64, 64, 20.0),
+                                            (1, 200, 255, 9.0)])
+def test_mlstm_single_token_kernel(dtype, H, dk, dv, cap):
+    """The one kernel for steps of single tokens against the four: the same maxima, outputs and states to rounding (the
+    compiler joins a product and a sum of the gates' arithmetic in one of them and not in the other)."""
+    ops = ops_for(dtype)
+    eps, slots, steps = 1e-5, [1, 3, 0], 4
+    n = len(slots) + 2
+    results = []
+    for fused in (False, True):
+        state = torch.zeros(4, H, dv + 1, dk, dtype=torch.float32, device=DEV)
+        maxima = torch.zeros(4, H, dtype=torch.float32, device=DEV)
+        outs = []
+        for step in range(steps):
+            packed, t = mlstm_setup(H, dk, dv, n, seed=70 + step, dtype=dtype)
+            if not fused:
+                outs.append(run_mlstm(ops, packed, t, H, dk, dv, cap, eps, state, maxima, [1] * 3, slots, pad_rows=2, pad_seqs=1).clone())
+                continue
+            tsq, cu, sl = step_ints([1] * 3, slots, 2, 1)
+            dev = {k: v.to(DEV) for k, v in t.items()}
+            out = torch.full((n, H * dv), 5.0, dtype=dtype, device=DEV)
+            assert ops.state_step(False, packed.to(DEV), H, H, dk, dv, dev["norm"], eps, state, tsq, cu, sl, 4, out,
+                                  i_bias=dev["i_bias"], f_bias=dev["f_bias"], cap=cap, max_state=maxima, denom_eps=plain.DENOM_EPS)
+            torch.cuda.synchronize()
+            outs.append(out.clone())
+        results.append((torch.cat(outs), state.clone(), maxima.clone()))
+    close(results[1][0], results[0][0].double(), 2e-6 if dtype == torch.float32 else 8e-3, "outputs")
+    close(results[1][1], results[0][1].double(), 2e-6, "states")
+    close(results[1][2], results[0][2].double(), 2e-6, "maxima")
+    assert float(results[1][1][2].abs().max()) == 0.0 and float(results[1][2][2].abs().max()) == 0.0     # slot 2 belongs to nobody
 
 
 def test_mlstm_first_tokens_use_the_floor_of_the_denominator():

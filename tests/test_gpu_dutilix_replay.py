@@ -9,7 +9,7 @@ import torch
 
 import trace_tools
 from dutilix_helpers import DUT, make_weights, plain_logits, plain_logits_bf16, plain_logits_f32, random_tokens
-from helpers import TOL_F32, bf16_tolerance, f32_tolerance, rel_err, write_model_dir
+from helpers import TOL_F32, bf16_tolerance, rel_err, write_model_dir
 
 pytestmark = pytest.mark.gpu
 
@@ -47,7 +47,10 @@ class Case:
                              for rid, toks in self.reqs.items() for p in range(len(toks)))
 
     def tol(self, dtype):
-        return f32_tolerance(self.f32_error) if dtype == "float32" else bf16_tolerance(self.bf16_error)
+        # float32: the usual bound, or eight times what 32-bit arithmetic alone does to the plain model (a case with a
+        # row that amplifies rounding a few hundred times shows it there too; another order of the same sums moves such a
+        # row by several times that)
+        return max(TOL_F32, 8 * self.f32_error) if dtype == "float32" else bf16_tolerance(self.bf16_error)
 
     def check(self, got, dtype, what):
         judge([rel_err(row, self.want[rid][pos]) for (rid, pos), row in got.items()], self.tol(dtype), dtype, what)
