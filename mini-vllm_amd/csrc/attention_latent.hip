@@ -90,13 +90,13 @@ extern "C" int mv_latent_prepare(const void* packed, long ld, int n, int QR, int
 // ---------------------------------------------------------------------------------------
 #define HL_TOKENS 8
 #define HL_MAX_IN 1024
-#define HL_COLS 64
-#define HL_SLICES 4
 
 // A workgroup takes HL_TOKENS rows, one head and HL_COLS output columns; its 256 threads are HL_COLS columns
 // times HL_SLICES slices of the inputs (slice s sums inputs s, s + HL_SLICES, ...), the slices are added in
-// order through LDS. The order of additions depends on IN alone.
-template <typename TIN, typename TOUT, typename TG>
+// order through LDS. (64 columns x 4 slices for steps of many rows; 16 x 16 for steps of few rows, whose few
+// workgroups a head would otherwise walk long runs of inputs one load after the other.) The order of additions
+// depends on IN and the variant.
+template <typename TIN, typename TOUT, typename TG, int HL_COLS, int HL_SLICES>
 __global__ void __launch_bounds__(256)
 head_linear_kernel(const TIN* __restrict__ x, long ldx, int ldx_head, WeightPtr w, int IN, int OUT, TOUT* __restrict__ y, long ldy,
                    int ldy_head, int tail, const float* __restrict__ table, const int* __restrict__ positions,
@@ -180,18 +180,27 @@ extern "C" int mv_head_linear(const void* x, long ldx, int ldx_head, const void*
     MV_REQUIRE((mode == 0 && !gate) || (mode == 1 && tail == 0), "head_linear: mode %d does not take these options", mode);
     if (n == 0) return 0;
     WeightPtr wp{w, weight_dtype};
-    dim3 grid((n + HL_TOKENS - 1) / HL_TOKENS, H, (OUT + HL_COLS - 1) / HL_COLS);
-    if (mode == 0) {
-        MV_DISPATCH_T(dtype, "head_linear",
-                      hipLaunchKernelGGL((head_linear_kernel<T, float, T>), grid, dim3(256), 0, stream, (const T*)x, ldx, ldx_head,
-                                         wp, IN, OUT, (float*)y, ldy, ldy_head, tail, table, positions, (const T*)nullptr, 0L,
-                                         token_seq, n));
-    } else {
-        MV_DISPATCH_T(dtype, "head_linear",
-                      hipLaunchKernelGGL((head_linear_kernel<float, T, T>), grid, dim3(256), 0, stream, (const float*)x, ldx,
-                                         ldx_head, wp, IN, OUT, (T*)y, ldy, ldy_head, 0, table, positions, (const T*)gate, ldg,
-                                         token_seq, n));
+    const bool few = n <= 64;
+    const int cols = few ? 16 : 64;
+    dim3 grid((n + HL_TOKENS - 1) / HL_TOKENS, H, (OUT + cols - 1) / cols);
+#define HL_LAUNCH(C, S)                                                                                                     \
+    if (mode == 0) {                                                                                                        \
+        MV_DISPATCH_T(dtype, "head_linear",                                                                                 \
+                      hipLaunchKernelGGL((head_linear_kernel<T, float, T, C, S>), grid, dim3(256), 0, stream, (const T*)x, ldx, \
+                                         ldx_head, wp, IN, OUT, (float*)y, ldy, ldy_head, tail, table, positions,           \
+                                         (const T*)nullptr, 0L, token_seq, n));                                             \
+    } else {                                                                                                                \
+        MV_DISPATCH_T(dtype, "head_linear",                                                                                 \
+                      hipLaunchKernelGGL((head_linear_kernel<float, T, T, C, S>), grid, dim3(256), 0, stream, (const float*)x,  \
+                                         ldx, ldx_head, wp, IN, OUT, (T*)y, ldy, ldy_head, 0, table, positions,             \
+                                         (const T*)gate, ldg, token_seq, n));                                               \
     }
+    if (few) {
+        HL_LAUNCH(16, 16)
+    } else {
+        HL_LAUNCH(64, 4)
+    }
+#undef HL_LAUNCH
     return mv_check_launch("head_linear");
 }
 

@@ -181,7 +181,7 @@ extern "C" int mv_moe_identity_add(void* y, long ldy, const void* h, long ldh, c
 }
 
 // float rows in place: x <- x * factor
-__global__ void scale_rows_kernel(float* __restrict__ x, long ld, int cols, long total, float factor) {
+__global__ void scale_f32_kernel(float* __restrict__ x, long ld, int cols, long total, float factor) {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     x[(i / cols) * ld + (i % cols)] *= factor;
@@ -191,6 +191,6 @@ extern "C" int mv_scale_f32(float* x, long ld, int rows, int cols, float factor,
     MV_REQUIRE(rows >= 0 && cols > 0 && ld >= cols && x, "scale: bad sizes rows=%d cols=%d", rows, cols);
     const long total = (long)rows * cols;
     if (total == 0) return 0;
-    hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, x, ld, cols, total, factor);
+    hipLaunchKernelGGL(scale_f32_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, x, ld, cols, total, factor);
     return mv_check_launch("scale");
 }

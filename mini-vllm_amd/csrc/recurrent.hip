@@ -910,18 +910,50 @@ state_scan_kernel(const float* __restrict__ qk, const float* __restrict__ vals, 
     float* S = state + (((size_t)state_slots[seq] * H + head) * DV + (live ? j : 0)) * (size_t)DK;
     float s[R];
     delta_state_io<R, false>(s, S, sub, DK, live);
+    // a run of tokens comes from memory into registers while the run before it is computed, and from there into LDS
+    // (loads are issued whatever the index, from clamped addresses, and dropped where they do not count)
+    constexpr int NQ = (TT * 2 * DPAD + 255) / 256;
+    constexpr int NV = (TT * COLS + 255) / 256;
+    float gq[NQ], gx[NV], gg = 0.f;
+    auto fetch = [&](int base) {
+        const int nt = min(TT, end - base);
+#pragma unroll
+        for (int x = 0; x < NQ; ++x) {
+            const int e = tid + x * 256;
+            const int tt = e / (2 * DPAD), rem = e % (2 * DPAD), a = rem / DPAD, i = rem % DPAD;
+            const bool ok = tt < nt && i < DK;
+            const float l = qk[(((size_t)(base + (tt < nt ? tt : 0)) * G + group) * 2 + a) * DK + (i < DK ? i : 0)];
+            gq[x] = ok ? l : 0.f;
+        }
+#pragma unroll
+        for (int x = 0; x < NV; ++x) {
+            const int e = tid + x * 256;
+            const int tt = e / COLS, jj = e % COLS;
+            const bool ok = tt < nt && j0 + jj < DV;
+            const float l = vals[((size_t)(base + (tt < nt ? tt : 0)) * H + head) * DV + (j0 + jj < DV ? j0 + jj : 0)];
+            gx[x] = ok ? l : 0.f;
+        }
+        if (tid < TT * 2) {
+            const int tt = tid / 2;
+            gg = gates[((size_t)(base + (tt < nt ? tt : 0)) * H + head) * 4 + tid % 2];
+        }
+    };
+    fetch(begin);
     for (int base = begin; base < end; base += TT) {
         const int nt = min(TT, end - base);
         __syncthreads();                                   // the run before has been read
-        for (int x = tid; x < nt * 2 * DPAD; x += 256) {
-            const int tt = x / (2 * DPAD), rem = x % (2 * DPAD), a = rem / DPAD, i = rem % DPAD;
-            sv[tt][a][i] = i < DK ? qk[(((size_t)(base + tt) * G + group) * 2 + a) * DK + i] : 0.f;
+#pragma unroll
+        for (int x = 0; x < NQ; ++x) {
+            const int e = tid + x * 256;
+            if (e < TT * 2 * DPAD) (&sv[0][0][0])[e] = gq[x];
         }
-        for (int x = tid; x < nt * COLS; x += 256) {
-            const int tt = x / COLS, jj = x % COLS;
-            sx[tt][jj] = j0 + jj < DV ? vals[((size_t)(base + tt) * H + head) * DV + j0 + jj] : 0.f;
+#pragma unroll
+        for (int x = 0; x < NV; ++x) {
+            const int e = tid + x * 256;
+            if (e < TT * COLS) (&sx[0][0])[e] = gx[x];
         }
-        if (tid < nt * 2) sg[tid / 2][tid % 2] = gates[((size_t)(base + tid / 2) * H + head) * 4 + tid % 2];
+        if (tid < TT * 2) sg[tid / 2][tid % 2] = gg;
+        if (base + TT < end) fetch(base + TT);             // in flight while this run is computed
         __syncthreads();
         for (int tt = 0; tt < nt; ++tt) {
             const float a = sg[tt][0], b = sg[tt][1], v = sx[tt][col];

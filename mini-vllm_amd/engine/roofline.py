@@ -55,6 +55,19 @@ KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
     "mv_soft_cap": (r"\bsoft_cap_kernel", None, 1),
     "mv_attention_sigmoid_ref": (r"\battention_sigmoid_kernel", None, 1),
     "mv_attention_prefill_sigmoid": (r"\battention_prefill_kernel", None, 1),
+    "mv_gdelta_prepare": (r"\bgdelta_prepare_kernel", r"\bconv_state_kernel", 2),
+    "mv_mlstm_prepare": (r"\bmlstm_gates_kernel", r"\bmlstm_prepare_kernel", 2),
+    "mv_state_scan": (r"\bstate_scan_kernel", None, 1),
+    "mv_state_finish": (r"\bstate_finish_kernel", None, 1),
+    "mv_state_step": (r"\bstate_step_kernel", r"\bconv_state_kernel", 2),
+    "mv_latent_prepare": (r"\blatent_prepare_kernel", None, 1),
+    "mv_head_linear": (r"\bhead_linear_kernel", None, 1),
+    "mv_attention_latent": (r"\battention_latent_kernel", None, 1),
+    "mv_attention_latent_split": (r"\battention_latent_split_kernel", r"\battention_latent_join_kernel", 2),
+    "mv_moe_route": (r"\bmoe_route_kernel", None, 1),
+    "mv_moe_swiglu_scale": (r"\bmoe_swiglu_scale_kernel", None, 1),
+    "mv_moe_identity_add": (r"\bmoe_identity_add_kernel", None, 1),
+    "mv_scale_f32": (r"\bscale_f32_kernel", None, 1),
 }
 _OURS = re.compile("|".join(f"(?:{p})" for spec in KERNELS_OF.values() for p in spec[:2] if p))
 
