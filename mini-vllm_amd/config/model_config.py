@@ -577,9 +577,10 @@ class DutilixConfig(ModelConfig):
             if kind == "delta":
                 kv_heads = m.get("kv_heads")
                 conv = m.get("conv")
+                # (taps not stated: the stored taps' shape states them, the loader fills them in; 0 stands for "not yet known")
                 mixer = DutilixMixer(type=kind, heads=heads, dim=dim, vdim=vdim,
                                      kv_heads=heads if kv_heads is None else _typed(kv_heads, "kv_heads", int, mw),
-                                     conv=1 if conv is None else _typed(conv, "conv", int, mw))
+                                     conv=0 if conv is None else _typed(conv, "conv", int, mw))
             elif kind == "mlstm":
                 mixer = DutilixMixer(type=kind, heads=heads, dim=dim, vdim=vdim,
                                      gate_cap=_require(m, "gate_cap", float, mw))
@@ -591,10 +592,13 @@ class DutilixConfig(ModelConfig):
                                       f"is rotated as a whole")
                 if rot is None and rot_dim:
                     raise ConfigError(f"{mw}: rot_dim {rot_dim} without a 'rot' section")
+                q_rank, kv_rank, scale = m.get("q_rank"), m.get("kv_rank"), m.get("scale")
+                # (ranks not stated: the stored norm weights' shapes state them, the loader fills them in)
                 mixer = DutilixMixer(type=kind, heads=heads, dim=dim, vdim=vdim, rot_dim=rot_dim,
                                      rot_base=10000.0 if rot is None else _require(rot, "base", float, mw + ".rot"),
-                                     q_rank=_require(m, "q_rank", int, mw), kv_rank=_require(m, "kv_rank", int, mw),
-                                     scale=_require(m, "scale", float, mw))
+                                     q_rank=0 if q_rank is None else _typed(q_rank, "q_rank", int, mw),
+                                     kv_rank=0 if kv_rank is None else _typed(kv_rank, "kv_rank", int, mw),
+                                     scale=(dim + rot_dim) ** -0.5 if scale is None else _typed(scale, "scale", float, mw))
             else:
                 raise ConfigError(f"{lw}: layer type {kind!r} is not supported (delta, mlstm, latent_attention)")
             mlp = _section(entry, "mlp", lw, optional=True)
@@ -659,13 +663,13 @@ class DutilixConfig(ModelConfig):
             if m.type == "delta":
                 if m.kv_heads <= 0 or m.heads % m.kv_heads:
                     raise ConfigError(f"{lw}: {m.heads} heads are not a multiple of {m.kv_heads} kv_heads")
-                if m.conv < 1:
+                if m.conv < 0:
                     raise ConfigError(f"{lw}: conv must be >= 1, got {m.conv}")
             elif m.type == "mlstm":
                 if not m.gate_cap > 0:
                     raise ConfigError(f"{lw}: gate_cap must be positive, got {m.gate_cap}")
             else:
-                if m.q_rank <= 0 or m.kv_rank <= 0:
+                if m.q_rank < 0 or m.kv_rank < 0:
                     raise ConfigError(f"{lw}: q_rank and kv_rank must be positive")
                 if m.rot_dim < 0 or m.rot_dim % 2:
                     raise ConfigError(f"{lw}: rot_dim {m.rot_dim} must be even and >= 0")

@@ -11,9 +11,10 @@ Tensor names on disk: ``embed``, ``head``, ``final.norm``; per layer i ``l<i>.no
 """
 from __future__ import annotations
 
+import dataclasses
 from typing import FrozenSet
 
-from ..config.model_config import DutilixConfig
+from ..config.model_config import ConfigError, DutilixConfig
 from ..parts.block import PreNormBlock, PreNormBlockSpec
 from ..parts.io import ScaledHeadSpec
 from ..parts.latent_attention import LatentAttentionSpec
@@ -34,6 +35,9 @@ def dutilix_plan(config: DutilixConfig) -> ModelPlan:
     layers, calls = [], []
     for i, l in enumerate(config.layers):
         m = l.mixer
+        if (m.type == "delta" and m.conv < 1) or (m.type == "latent_attention" and (m.q_rank < 1 or m.kv_rank < 1)):
+            raise ValueError(f"layer {i}: config.json states no taps (delta) or ranks (latent_attention); the stored "
+                             f"tensors do (see dutilix_complete)")
         if m.type == "delta":
             mixer = GatedDeltaSpec(hidden_size=hid, num_heads=m.heads, num_kv_heads=m.kv_heads, key_dim=m.dim,
                                    value_dim=m.vdim, conv_taps=m.conv, unit_eps=1e-6, out_norm_eps=eps)
@@ -102,10 +106,35 @@ def dutilix_ignorable(config: DutilixConfig) -> FrozenSet[str]:
     return frozenset(f"l{i}.norm2" for i, l in enumerate(config.layers) if l.mlp is None)
 
 
+def dutilix_complete(config: DutilixConfig, source) -> DutilixConfig:
+    """The configuration with what only the stored tensors state, where config.json leaves it out: a delta layer's taps
+    are the columns of ``l<i>.mix.q.conv``, an attention layer's ranks the lengths of ``l<i>.mix.dq.norm`` and
+    ``l<i>.mix.dkv.norm``."""
+    names = set(source.names())
+
+    def length(name: str, axis: int) -> int:
+        if name not in names or len(source.shape(name)) <= axis:
+            raise ConfigError(f"the model has no tensor {name!r}, which states a size that config.json leaves out")
+        return int(source.shape(name)[axis])
+
+    layers = []
+    for i, l in enumerate(config.layers):
+        m = l.mixer
+        if m.type == "delta" and m.conv < 1:
+            m = dataclasses.replace(m, conv=length(f"l{i}.mix.q.conv", 1))
+        if m.type == "latent_attention" and m.q_rank < 1:
+            m = dataclasses.replace(m, q_rank=length(f"l{i}.mix.dq.norm", 0))
+        if m.type == "latent_attention" and m.kv_rank < 1:
+            m = dataclasses.replace(m, kv_rank=length(f"l{i}.mix.dkv.norm", 0))
+        layers.append(dataclasses.replace(l, mixer=m))
+    return dataclasses.replace(config, layers=tuple(layers))
+
+
 DUTILIX = register_architecture(Architecture(
     name=DutilixConfig.architecture,
     config_class=DutilixConfig,
     plan=dutilix_plan,
     tensor_name=dutilix_tensor_name,
     ignorable=dutilix_ignorable,
+    complete=dutilix_complete,
 ))

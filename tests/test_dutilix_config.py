@@ -39,7 +39,7 @@ def test_defaults_and_optional_keys():
 @pytest.mark.parametrize("edit, message", [
     (lambda c: c["layers"][0].update(type="conv"), "not supported"),
     (lambda c: c["layers"][0]["mixer"].update(kv_heads=3), "multiple"),
-    (lambda c: c["layers"][0]["mixer"].update(conv=0), "conv"),
+    (lambda c: c["layers"][0]["mixer"].update(conv=-2), "conv"),
     (lambda c: c["layers"][0]["mlp"]["router"]["groups"].update(count=4), "groups"),
     (lambda c: c["layers"][0]["mlp"]["router"].update(top=7), "top"),
     (lambda c: c["layers"][1]["mixer"]["rot"].update(dims=4), "rot.dims"),
@@ -127,3 +127,23 @@ def test_plain_short_convolution_edges():
     assert torch.equal(y2, y[4:]) and torch.equal(kept2, kept)
     y1, kept1 = plain.short_conv(x[:1], taps)
     assert torch.equal(kept1, torch.stack([torch.zeros(2, dtype=torch.float64), x[0]]))
+
+
+def test_sizes_that_config_json_leaves_out_come_from_the_tensors():
+    """Taps, both ranks and the attention's scale may be absent: taps and ranks are read off the stored tensors'
+    shapes, the scale is (dim + rot_dim)^-1/2."""
+    from minivllm_amd.weights.source import DictSource
+    cfg = copy.deepcopy(DUT_A)
+    del cfg["layers"][0]["mixer"]["conv"]
+    for key in ("q_rank", "kv_rank", "scale"):
+        del cfg["layers"][1]["mixer"][key]
+    arch, bare = load(cfg)
+    with pytest.raises(ValueError, match="taps"):
+        arch.plan(bare)
+    weights = make_weights(DUT_A, seed=1)
+    full = arch.complete(bare, DictSource(weights))
+    _, want = load(DUT_A)
+    assert full.layers[0] == want.layers[0] and full.layers[2:] == want.layers[2:]
+    got, ref = full.layers[1].mixer, want.layers[1].mixer
+    assert (got.q_rank, got.kv_rank) == (ref.q_rank, ref.kv_rank) and abs(got.scale - (16 + 8) ** -0.5) < 1e-12
+    arch.plan(full)
