@@ -194,3 +194,197 @@ extern "C" int mv_scale_f32(float* x, long ld, int rows, int cols, float factor,
     hipLaunchKernelGGL(scale_f32_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, x, ld, cols, total, factor);
     return mv_check_launch("scale");
 }
+
+#ifdef MV_WITH_BF16
+// =======================================================================================
+// The experts' products over the chosen (token, expert) pairs only (bfloat16, MFMA).
+//
+//   moe_sort      counts the pairs of every expert, lays the pairs out expert by expert (`sorted`: pair
+//                 indices, a pair is token * top + place) and cuts every expert's run into tiles of 64 rows
+//                 (`tile_expert`, `tile_row0`, `tile_rows`; unused entries hold expert -1). Identity experts
+//                 and pairs without an expert are left out. Within an expert the order of the pairs is
+//                 whatever the counters gave; no result depends on it (a row's products read only its own row).
+//   moe_gate_up   per tile and 128 columns: act[pair] = weight[pair] * silu(x W_gate^T) * (x W_up^T), the rows of x
+//                 gathered through `sorted`, rounded once
+//   moe_down      per tile and 128 columns: out[pair] = act[pair] W_down^T as floats
+//   moe_combine   y[token] = sum over its places (in order) of out[pair] + (identity weights) * x[token]
+//
+// A workgroup takes a tile and 128 columns; each of its four waves computes 16 rows x 128 columns (x 2 for gate and
+// up) with v_mfma_f32_16x16x32_bf16: lane l holds row l % 16 of the first operand (8 values of k from 8 (l / 16))
+// and column l % 16 of the second, and ends with column l % 16 of rows 4 (l / 16) .. + 3. The four waves read the
+// same weight rows, which the caches serve; a weight is read once for 64 rows. K must be a multiple of 32 and rows
+// 16-byte aligned.
+// =======================================================================================
+typedef __bf16 mg_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float mg_f4 __attribute__((ext_vector_type(4)));
+union MgFrag {
+    uint4 u;
+    mg_bf16x8 v;
+};
+#define MG_ROWS 64             // rows of a tile: four waves of 16 rows each
+#define MG_COLS 128            // columns of a workgroup (gate columns, with their up columns, when gated)
+
+__global__ void __launch_bounds__(1024)
+moe_sort_kernel(const int* __restrict__ ids, int n_pairs, int n_real, int max_tiles, int* __restrict__ sorted,
+                int* __restrict__ tile_expert, int* __restrict__ tile_row0, int* __restrict__ tile_rows) {
+    __shared__ int count[MR_MAX_E], offset[MR_MAX_E], cursor[MR_MAX_E];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < n_real; e += 1024) {
+        count[e] = 0;
+        cursor[e] = 0;
+    }
+    __syncthreads();
+    for (int p = tid; p < n_pairs; p += 1024) {
+        const int e = ids[p];
+        if (e >= 0 && e < n_real) atomicAdd(&count[e], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int off = 0, t = 0;
+        for (int e = 0; e < n_real; ++e) {
+            offset[e] = off;
+            const int c = count[e];
+            for (int r = 0; r < c && t < max_tiles; r += MG_ROWS, ++t) {
+                tile_expert[t] = e;
+                tile_row0[t] = off + r;
+                tile_rows[t] = min(MG_ROWS, c - r);
+            }
+            off += c;
+        }
+        for (; t < max_tiles; ++t) tile_expert[t] = -1;
+    }
+    __syncthreads();
+    for (int p = tid; p < n_pairs; p += 1024) {
+        const int e = ids[p];
+        if (e >= 0 && e < n_real) sorted[offset[e] + atomicAdd(&cursor[e], 1)] = p;
+    }
+}
+
+// GATED: W holds [E gate blocks of F rows | E up blocks of F rows], K columns each (ldw = K); the output is the
+// weighted activation. Otherwise W is [N rows][ldw] with the expert's K columns from column e * K (all down
+// matrices side by side); the output is float.
+template <bool GATED>
+__global__ void __launch_bounds__(256)
+moe_expert_product_kernel(const bf16* __restrict__ a, long lda, int a_by_token, const bf16* __restrict__ w, long ldw, int E, int N,
+                          int K, const int* __restrict__ sorted, const int* __restrict__ tile_expert,
+                          const int* __restrict__ tile_row0, const int* __restrict__ tile_rows, const float* __restrict__ weights,
+                          int top, bf16* __restrict__ act, float* __restrict__ out) {
+    const int tile = blockIdx.x;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int row0 = tile_row0[tile] + 16 * wave, nrows = tile_rows[tile] - 16 * wave;     // this wave's 16 rows
+    if (nrows <= 0) return;
+    const int r = lane % 16, kq = lane / 16;
+    const int pair = r < nrows ? sorted[row0 + r] : -1;
+    const bf16* arow = pair < 0 ? nullptr : a + (size_t)(a_by_token ? pair / top : pair) * lda;
+    const int n0 = blockIdx.y * MG_COLS;
+    constexpr int NS = MG_COLS / 16;
+    const bf16* b0[NS];
+    const bf16* b1[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const int col = n0 + 16 * s + r;
+        const int c = col < N ? col : N - 1;               // columns past the end: some column; never stored
+        if (GATED) {
+            b0[s] = w + ((size_t)e * N + c) * ldw;
+            b1[s] = w + ((size_t)(E + e) * N + c) * ldw;
+        } else {
+            b0[s] = w + (size_t)c * ldw + (size_t)e * K;
+            b1[s] = b0[s];
+        }
+    }
+    mg_f4 acc0[NS], acc1[GATED ? NS : 1];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) acc0[s] = mg_f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < (GATED ? NS : 1); ++s) acc1[s] = mg_f4{0.f, 0.f, 0.f, 0.f};
+    const uint4 zero = uint4{0u, 0u, 0u, 0u};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const int kk = k0 + 8 * kq;
+        MgFrag fa, fb[NS], fc[GATED ? NS : 1];
+        fa.u = arow ? *reinterpret_cast<const uint4*>(arow + kk) : zero;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            fb[s].u = *reinterpret_cast<const uint4*>(b0[s] + kk);
+            if (GATED) fc[s].u = *reinterpret_cast<const uint4*>(b1[s] + kk);
+        }
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            acc0[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa.v, fb[s].v, acc0[s], 0, 0, 0);
+            if (GATED) acc1[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa.v, fc[s].v, acc1[s], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int idx = 0; idx < 4; ++idx) {
+        const int i = 4 * kq + idx;
+        if (i >= nrows) continue;
+        const int p = sorted[row0 + i];
+        const float wt = GATED ? weights[p] : 0.f;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const int col = n0 + 16 * s + r;
+            if (col >= N) continue;
+            if (GATED) {
+                const float g = acc0[s][idx], u = acc1[s][idx];
+                act[(size_t)p * N + col] = from_f<bf16>(wt * (g / (1.f + expf(-g))) * u);
+            } else {
+                out[(size_t)p * N + col] = acc0[s][idx];
+            }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+moe_combine_kernel(const float* __restrict__ out, const int* __restrict__ ids, int top, int n_real, const bf16* __restrict__ x,
+                   long ldx, const float* __restrict__ dense, int ld_dense, int identity, bf16* __restrict__ y, long ldy, int width) {
+    const int t = blockIdx.x;
+    float idw = 0.f;
+    for (int e = 0; e < identity; ++e) idw += dense[(size_t)t * ld_dense + n_real + e];
+    for (int c = threadIdx.x; c < width; c += 256) {
+        float v = 0.f;
+        for (int k = 0; k < top; ++k) {
+            const int e = ids[(size_t)t * top + k];
+            if (e >= 0 && e < n_real) v += out[((size_t)t * top + k) * width + c];
+        }
+        if (idw != 0.f) v = fmaf(idw, to_f(x[(size_t)t * ldx + c]), v);
+        y[(size_t)t * ldy + c] = from_f<bf16>(v);
+    }
+}
+
+// ints of scratch: sorted pairs and the three tile tables; floats: the down products of every pair
+extern "C" long mv_moe_grouped_ints(int n, int top, int n_real) { return (long)n * top + 3L * ((long)n * top / MG_ROWS + n_real + 1); }
+
+// returns 2 (nothing done) for sizes it does not serve
+extern "C" int mv_moe_grouped(const void* x, long ldx, int n, int hidden, const void* w_gate_up, const void* w_down, int n_real,
+                              int identity, int F, const int* ids, const float* weights, int top, const float* dense,
+                              int ld_dense, int* ints, void* act, float* out, void* y, long ldy, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && hidden > 0 && n_real > 0 && F > 0 && top > 0 && identity >= 0, "moe_grouped: bad sizes");
+    if (hidden % 32 || F % 32 || ldx % 8 || ((uintptr_t)x % 16) || ((uintptr_t)w_gate_up % 16) || ((uintptr_t)w_down % 16)
+        || ((uintptr_t)act % 16) || n_real > MR_MAX_E)
+        return 2;
+    MV_REQUIRE(x && w_gate_up && w_down && ids && weights && dense && ints && act && out && y && ld_dense >= n_real + identity
+               && ldy >= hidden, "moe_grouped: missing operand");
+    if (n == 0) return 0;
+    const int n_pairs = n * top;
+    const int max_tiles = n_pairs / MG_ROWS + n_real + 1;
+    int* sorted = ints;
+    int* tile_expert = ints + n_pairs;
+    int* tile_row0 = tile_expert + max_tiles;
+    int* tile_rows = tile_row0 + max_tiles;
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, n_pairs, n_real, max_tiles, sorted, tile_expert,
+                       tile_row0, tile_rows);
+    if (mv_check_launch("moe_sort")) return 1;
+    hipLaunchKernelGGL(moe_expert_product_kernel<true>, dim3(max_tiles, (F + MG_COLS - 1) / MG_COLS), dim3(256), 0, stream, (const bf16*)x, ldx,
+                       1, (const bf16*)w_gate_up, (long)hidden, n_real, F, hidden, sorted, tile_expert, tile_row0, tile_rows,
+                       weights, top, (bf16*)act, (float*)nullptr);
+    if (mv_check_launch("moe_gate_up")) return 1;
+    hipLaunchKernelGGL(moe_expert_product_kernel<false>, dim3(max_tiles, (hidden + MG_COLS - 1) / MG_COLS), dim3(256), 0, stream,
+                       (const bf16*)act, (long)F, 0, (const bf16*)w_down, (long)n_real * F, n_real, hidden, F, sorted, tile_expert,
+                       tile_row0, tile_rows, weights, top, (bf16*)nullptr, out);
+    if (mv_check_launch("moe_down")) return 1;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(n), dim3(256), 0, stream, out, ids, top, n_real, (const bf16*)x, ldx, dense,
+                       ld_dense, identity, (bf16*)y, ldy, hidden);
+    return mv_check_launch("moe_combine");
+}
+#endif

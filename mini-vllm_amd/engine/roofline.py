@@ -68,6 +68,7 @@ KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
     "mv_moe_swiglu_scale": (r"\bmoe_swiglu_scale_kernel", None, 1),
     "mv_moe_identity_add": (r"\bmoe_identity_add_kernel", None, 1),
     "mv_scale_f32": (r"\bscale_f32_kernel", None, 1),
+    "mv_moe_grouped": (r"\bmoe_sort_kernel", r"\bmoe_(expert_product|combine)_kernel", 4),
 }
 _OURS = re.compile("|".join(f"(?:{p})" for spec in KERNELS_OF.values() for p in spec[:2] if p))
 

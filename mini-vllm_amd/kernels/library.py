@@ -82,6 +82,10 @@ _SIGNATURES = {
 
 # entry points that only the bfloat16 library has
 _OPTIONAL_SIGNATURES = {
+    "mv_moe_grouped_ints": (c_long, [c_int, c_int, c_int]),
+    # x, ldx, n, hidden, w_gate_up, w_down, n_real, identity, F, ids, weights, top, dense, ld_dense, ints, act, out, y, ldy, stream
+    "mv_moe_grouped": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int,
+                               c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p]),
     "mv_gemm_skinny": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int,
                                c_int, c_int, c_int, c_void_p]),
     "mv_gemm_skinny_swiglu": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p]),

@@ -901,6 +901,41 @@ class Ops:
                       h.stride(0) if n > 1 else width, dense.data_ptr(), dense.stride(0) if n > 1 else dense.shape[1], first,
                       count, n, width, int(overwrite), self.code, self._stream())
 
+    def moe_grouped(self, x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, experts: int, identity: int, ff: int,
+                    ids: torch.Tensor, weights: torch.Tensor, dense: torch.Tensor, ints: torch.Tensor, act: torch.Tensor,
+                    out: torch.Tensor, y: torch.Tensor) -> bool:
+        """The experts' products over the chosen (token, expert) pairs only (bfloat16): y[t] = sum over t's chosen experts
+        of weight * down_e(silu(gate_e x) * up_e x) + (its identity experts' weights) * x[t]. ``w_gate_up`` is
+        [2 * experts * ff, hidden] (all gate blocks, then all up blocks), ``w_down`` [hidden, experts * ff]; ids / weights
+        [n, top] and dense [n, experts + identity] as ``moe_route`` leaves them; ``ints`` (int32), ``act`` [n * top, ff]
+        and ``out`` float32 [n * top, hidden] are scratch. False when the sizes are not served (nothing was done)."""
+        if self.dtype != torch.bfloat16 or not self.lib.has("mv_moe_grouped") or w_gate_up.dtype != torch.bfloat16 \
+                or w_down.dtype != torch.bfloat16:
+            return False
+        self._act(x, "feed-forward input"); self._act(y, "feed-forward output"); self._act(act, "expert activations")
+        n, hidden = x.shape
+        top = ids.shape[1]
+        if tuple(w_gate_up.shape) != (2 * experts * ff, hidden) or tuple(w_down.shape) != (hidden, experts * ff) \
+                or not w_gate_up.is_contiguous() or not w_down.is_contiguous() or x.stride(1) != 1 or y.stride(1) != 1 \
+                or tuple(y.shape) != (n, hidden) or tuple(act.shape) != (n * top, ff) or not act.is_contiguous() \
+                or out.dtype != torch.float32 or tuple(out.shape) != (n * top, hidden) or not out.is_contiguous() \
+                or ids.dtype != torch.int32 or tuple(weights.shape) != (n, top) or weights.dtype != torch.float32 \
+                or not ids.is_contiguous() or not weights.is_contiguous() or dense.dtype != torch.float32 \
+                or dense.shape[0] != n or dense.shape[1] < experts + identity or dense.stride(1) != 1 \
+                or ints.dtype != torch.int32 or ints.numel() < int(self.lib.dll.mv_moe_grouped_ints(n, top, experts)):
+            raise KernelLibraryError("moe_grouped: operands do not fit")
+        for t in (w_gate_up, w_down, ids, weights, dense, ints, out):
+            _dev(t, "moe_grouped operand")
+        if not self.lib.offer("mv_moe_grouped", x.data_ptr(), x.stride(0) if n > 1 else hidden, n, hidden, w_gate_up.data_ptr(),
+                              w_down.data_ptr(), experts, identity, ff, ids.data_ptr(), weights.data_ptr(), top, dense.data_ptr(),
+                              dense.stride(0) if n > 1 else dense.shape[1], ints.data_ptr(), act.data_ptr(), out.data_ptr(),
+                              y.data_ptr(), y.stride(0) if n > 1 else hidden, self._stream()):
+            return False
+        used = min(experts, n * top)
+        self._note("mv_moe_grouped", self._size(x, y) + used * 3 * ff * hidden * 2 + self._size(act, out) * 2,
+                   2 * n * top * 3 * ff * hidden)
+        return True
+
     def scale_f32(self, x: torch.Tensor, factor: float) -> None:
         """In place on float32 [rows, cols]: x <- x * factor."""
         _dev(x, "rows")

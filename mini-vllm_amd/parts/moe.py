@@ -9,10 +9,15 @@ largest (outputs of other groups cannot be chosen whatever their number). The we
 experts' scores divided by their sum (+ weight_sum_eps); the result is the weighted sum of the
 chosen experts' outputs.
 
-How it runs: gate and up matrices of all experts form one packed product and all down matrices one
-second product; between them one kernel applies SiLU, the up factor and the router's weight (zero
-for experts that were not chosen) before the single rounding, so the second product sums exactly the
-chosen experts. Everything is decided on the device; nothing about a step's routing reaches the host.
+How it runs. In bfloat16, when the sizes allow (``grouped``): the chosen (token, expert) pairs are sorted
+by expert on the device, every expert's pairs are cut into tiles of 64 rows, and two MFMA kernels compute
+gate/up with the weighted activation and the down product for those tiles only; a last kernel sums a
+token's pairs in the order of choice and adds the identity experts' share. Otherwise (float32, odd
+sizes): gate and up matrices of all experts form one packed product and all down matrices one second
+product; between them one kernel applies SiLU, the up factor and the router's weight (zero for experts
+that were not chosen) before the single rounding, so the second product sums exactly the chosen
+experts. Either way everything is decided on the device; nothing about a step's routing reaches the
+host, so steps replay from graphs.
 """
 from __future__ import annotations
 
@@ -36,6 +41,9 @@ class RoutedExpertsSpec(PartSpec):
     keep_groups: int = 1
     correction: bool = False             # a stored number per router output added to the scores for the choice
     weight_sum_eps: float = 1e-20
+    grouped: bool = True                 # bfloat16: the experts' products over the chosen pairs only, where the sizes allow
+    grouped_min_rows: int = 16           # ... from this many chosen rows an expert on average (steps of fewer rows stream
+                                         # every expert's weights once, which their few rows cannot beat)
 
     @property
     def router_outputs(self) -> int:
@@ -87,6 +95,13 @@ class RoutedExperts(FeedForward):
         weights = ws.get("moe.weights", (n, spec.top), torch.float32)
         ops.moe_route(logits, self.correction, spec.groups, spec.keep_groups, spec.top, spec.weight_sum_eps, dense, ids, weights)
         y = ws.get("ffn.out", (n, spec.hidden_size), rt.dtype)
+        if n_e and spec.grouped and ops.use_fast_kernels and n * spec.top >= spec.grouped_min_rows * n_e:
+            # the chosen (token, expert) pairs only: sorted by expert on the device, tiles of 64 rows through MFMA
+            need = int(ops.lib.dll.mv_moe_grouped_ints(n, spec.top, n_e)) if ops.lib.has("mv_moe_grouped") else 0
+            if need and ops.moe_grouped(x, self.w_gate_up, self.w_down, n_e, spec.identity_experts, F, ids, weights, dense,
+                                        ws.get("moe.ints", (need,), torch.int32), ws.get("moe.pair_act", (n * spec.top, F), rt.dtype),
+                                        ws.get("moe.pair_out", (n * spec.top, spec.hidden_size), torch.float32), y):
+                return y
         if n_e:
             gu = ws.get("moe.gate_up", (n, 2 * n_e * F), rt.dtype)
             ops.gemm(x, self.w_gate_up, gu)

@@ -634,6 +634,43 @@ def test_routed_experts_against_the_plain_mixture(dtype):
     close(got, want, 3e-5 if dtype == torch.float32 else 2e-2, "mixture")
 
 
+@pytest.mark.parametrize("n", [1, 7, 70, 300])
+@pytest.mark.parametrize("hid, F, E, I, top, groups, keep", [(64, 32, 5, 3, 3, 4, 3), (96, 64, 16, 0, 4, 4, 2), (32, 160, 3, 1, 4, 1, 1)])
+def test_grouped_experts_against_all_experts(n, hid, F, E, I, top, groups, keep):
+    """bfloat16 with sizes the MFMA kernels serve: the products over the chosen pairs only give what computing every
+    expert and zeroing the others gives, and what the plain mixture gives."""
+    from minivllm_amd.parts.base import Runtime, Workspace
+    from minivllm_amd.parts.moe import RoutedExperts, RoutedExpertsSpec
+    dtype = torch.bfloat16
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(n + E)
+    w = {"router": 3.0 * torch.randn(E + I, hid, generator=g) / hid ** 0.5, "correction": 0.05 * torch.randn(E + I, generator=g)}
+    for e in range(E):
+        w[f"e{e}.gate"] = torch.randn(F, hid, generator=g) / hid ** 0.5
+        w[f"e{e}.up"] = torch.randn(F, hid, generator=g) / hid ** 0.5
+        w[f"e{e}.down"] = torch.randn(hid, F, generator=g) / F ** 0.5
+    w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    tensors = {"router": w["router"].to(DEV), "correction": w["correction"].to(DEV)}
+    for e in range(E):
+        for k in ("gate", "up", "down"):
+            tensors[f"{k}.{e}"] = w[f"e{e}.{k}"].to(DEV)
+    x = torch.randn(n, hid, generator=g).to(dtype)
+    outs = {}
+    for grouped in (True, False):
+        spec = RoutedExpertsSpec(hidden_size=hid, expert_size=F, num_experts=E, identity_experts=I, top=top, groups=groups,
+                                 keep_groups=keep, correction=True, grouped=grouped, grouped_min_rows=0)
+        rt = Runtime(device=torch.device(DEV), dtype=dtype, ops=ops, workspace=Workspace(torch.device(DEV)), max_positions=64)
+        ops.ledger = []
+        outs[grouped] = RoutedExperts(spec, tensors, rt).forward(x.to(DEV), None).clone()
+        torch.cuda.synchronize()
+        assert ("mv_moe_grouped" in [e[0] for e in ops.ledger]) == grouped
+        ops.ledger = None
+    mlp = {"kind": "moe", "expert": {"ff": F}, "router": {"experts": E, "identity": I, "top": top, "groups": {"count": groups, "keep": keep}}}
+    want = plain.mixture(x.double(), {"m." + k: v.double() for k, v in w.items()}, "m.", mlp)
+    close(outs[True], want, 2e-2, "chosen pairs only against the plain mixture")
+    close(outs[True], outs[False].double(), 2e-2, "chosen pairs only against all experts")
+
+
 def test_scaled_logits():
     ops = ops_for(torch.float32)
     x = torch.randn(5, 33, device=DEV)
