@@ -9,15 +9,21 @@ largest (outputs of other groups cannot be chosen whatever their number). The we
 experts' scores divided by their sum (+ weight_sum_eps); the result is the weighted sum of the
 chosen experts' outputs.
 
-How it runs. In bfloat16, when the sizes allow (``grouped``): the chosen (token, expert) pairs are sorted
-by expert on the device, every expert's pairs are cut into tiles of 64 rows, and two MFMA kernels compute
-gate/up with the weighted activation and the down product for those tiles only; a last kernel sums a
-token's pairs in the order of choice and adds the identity experts' share. Otherwise (float32, odd
-sizes): gate and up matrices of all experts form one packed product and all down matrices one second
-product; between them one kernel applies SiLU, the up factor and the router's weight (zero for experts
-that were not chosen) before the single rounding, so the second product sums exactly the chosen
-experts. Either way everything is decided on the device; nothing about a step's routing reaches the
-host, so steps replay from graphs.
+How it runs: gate and up matrices of all experts form one packed product and all down matrices one
+second product; between them one kernel applies SiLU, the up factor and the router's weight (zero
+for experts that were not chosen) before the single rounding, so the second product sums exactly the
+chosen experts. That is exact, replays from graphs and runs at the library product's rate, but computes
+every expert: eight times the useful multiply-adds when a token uses an eighth of the experts, and every
+expert's bytes in a decode step. With ``grouped`` (bfloat16, widths that are multiples of 32) the chosen
+(token, expert) pairs are instead sorted by expert on the device, every expert's pairs are cut into tiles
+of 64 rows, and two MFMA kernels compute gate/up with the weighted activation and the down product for
+those tiles only; a last kernel sums a token's pairs in the order of choice and adds the identity experts'
+share. Its plain MFMA kernels (operands straight from memory) win where bytes decide, steps of few rows
+against large experts (8B-sized layers, 32 experts, 4 a token: a step of one request 8.8 against 13.1 ms,
+of eight 12.2 against 13.4), and lose or draw elsewhere (0.6B-sized layers at eight requests 3.0 against
+2.4 ms; a prompt of 2,048 tokens 440 against 465 us a layer at 0.6B sizes, but 186 against 151 ms for the
+whole prompt at 8B sizes), so the spec's thresholds send only the former there. Either way everything is decided on the device;
+nothing about a step's routing reaches the host, so steps replay from graphs.
 """
 from __future__ import annotations
 
@@ -41,9 +47,12 @@ class RoutedExpertsSpec(PartSpec):
     keep_groups: int = 1
     correction: bool = False             # a stored number per router output added to the scores for the choice
     weight_sum_eps: float = 1e-20
-    grouped: bool = True                 # bfloat16: the experts' products over the chosen pairs only, where the sizes allow
-    grouped_min_rows: int = 16           # ... from this many chosen rows an expert on average (steps of fewer rows stream
-                                         # every expert's weights once, which their few rows cannot beat)
+    # bfloat16, widths that are multiples of 32: the experts' products over the chosen (token, expert) pairs only, in steps
+    # with fewer than ``grouped_max_rows`` chosen rows an expert on average and experts of at least ``grouped_min_weight``
+    # elements a matrix (there a step is bound by the bytes of the experts it reads, and most experts are not chosen)
+    grouped: bool = True
+    grouped_max_rows: float = 2.0
+    grouped_min_weight: int = 4 * 1024 * 1024
 
     @property
     def router_outputs(self) -> int:
@@ -83,6 +92,12 @@ class RoutedExperts(FeedForward):
                                        + [tensors[f"up.{e}"] for e in range(n_e)], dim=0).contiguous()
             self.w_down = torch.cat([tensors[f"down.{e}"] for e in range(n_e)], dim=1).contiguous()
 
+    def wants_grouped(self, n: int) -> bool:
+        """Whether a step of n rows computes the chosen pairs only (where the kernels take the sizes)."""
+        spec = self.spec
+        return (spec.grouped and n * spec.top < spec.grouped_max_rows * spec.num_experts
+                and spec.expert_size * spec.hidden_size >= spec.grouped_min_weight)
+
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
         if not isinstance(x, torch.Tensor):
@@ -95,7 +110,7 @@ class RoutedExperts(FeedForward):
         weights = ws.get("moe.weights", (n, spec.top), torch.float32)
         ops.moe_route(logits, self.correction, spec.groups, spec.keep_groups, spec.top, spec.weight_sum_eps, dense, ids, weights)
         y = ws.get("ffn.out", (n, spec.hidden_size), rt.dtype)
-        if n_e and spec.grouped and ops.use_fast_kernels and n * spec.top >= spec.grouped_min_rows * n_e:
+        if n_e and ops.use_fast_kernels and self.wants_grouped(n):
             # the chosen (token, expert) pairs only: sorted by expert on the device, tiles of 64 rows through MFMA
             need = int(ops.lib.dll.mv_moe_grouped_ints(n, spec.top, n_e)) if ops.lib.has("mv_moe_grouped") else 0
             if need and ops.moe_grouped(x, self.w_gate_up, self.w_down, n_e, spec.identity_experts, F, ids, weights, dense,

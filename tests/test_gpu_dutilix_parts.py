@@ -658,7 +658,7 @@ def test_grouped_experts_against_all_experts(n, hid, F, E, I, top, groups, keep)
     outs = {}
     for grouped in (True, False):
         spec = RoutedExpertsSpec(hidden_size=hid, expert_size=F, num_experts=E, identity_experts=I, top=top, groups=groups,
-                                 keep_groups=keep, correction=True, grouped=grouped, grouped_min_rows=0)
+                                 keep_groups=keep, correction=True, grouped=grouped, grouped_max_rows=1e9, grouped_min_weight=0)
         rt = Runtime(device=torch.device(DEV), dtype=dtype, ops=ops, workspace=Workspace(torch.device(DEV)), max_positions=64)
         ops.ledger = []
         outs[grouped] = RoutedExperts(spec, tensors, rt).forward(x.to(DEV), None).clone()
