@@ -9,7 +9,8 @@
 //                        the way; weighted latents into values, times the output gate)
 //     attention_latent   softmax attention with one shared key row of R + DR numbers whose first R
 //                        are also the value
-// Page layout: rows[page][slot][R + DR] in the activation type. Scores, weights and sums are float.
+// Page layout: rows[page][slot][R + DR] in the activation type, and the latents once more with a page's slots side
+// by side, [page][R][slot], which is how the MFMA kernel's second product wants them. Scores, weights and sums are float.
 #include "dispatch.h"
 
 // ---------------------------------------------------------------------------------------
@@ -23,7 +24,7 @@ __global__ void __launch_bounds__(256)
 latent_prepare_kernel(const T* __restrict__ packed, long ld, int QR, int R, int DR, WeightPtr wq, WeightPtr wkv, float eps,
                       const float* __restrict__ table, const int* __restrict__ positions, const int* __restrict__ token_seq,
                       const int* __restrict__ block_table, int bt_width, int page_size, T* __restrict__ cq, long ldq,
-                      T* __restrict__ pages) {
+                      T* __restrict__ pages, T* __restrict__ pages_t) {
     __shared__ float scratch[17];
     const int t = blockIdx.x, tid = threadIdx.x;
     const int seq = token_seq[t];
@@ -52,7 +53,13 @@ latent_prepare_kernel(const T* __restrict__ packed, long ld, int QR, int R, int 
     const int pos = positions[t];
     const int page = block_table[(size_t)seq * bt_width + pos / page_size];
     T* row = pages + ((size_t)page * page_size + pos % page_size) * (size_t)(R + DR);
-    for (int c = tid; c < R; c += 256) row[c] = from_f<T>(to_f(kv[c]) * inv * wkv.at(c));
+    // (pages_t, when given, holds the latent once more with the slots of a page side by side: [page][R][slot])
+    T* col = pages_t ? pages_t + (size_t)page * R * page_size + pos % page_size : nullptr;
+    for (int c = tid; c < R; c += 256) {
+        const T v = from_f<T>(to_f(kv[c]) * inv * wkv.at(c));
+        row[c] = v;
+        if (col) col[(size_t)c * page_size] = v;
+    }
     const int half = DR / 2;
     const float* cs = table + (size_t)pos * DR;
     for (int i = tid; i < half; i += 256) {
@@ -66,7 +73,7 @@ latent_prepare_kernel(const T* __restrict__ packed, long ld, int QR, int R, int 
 extern "C" int mv_latent_prepare(const void* packed, long ld, int n, int QR, int R, int DR, const void* wq, const void* wkv,
                                  int weight_dtype, float eps, const float* table, int table_rows, const int* positions,
                                  const int* token_seq, const int* block_table, int bt_width, int page_size, void* cq,
-                                 long ldq, void* pages, int dtype, hipStream_t stream) {
+                                 long ldq, void* pages, void* pages_t, int dtype, hipStream_t stream) {
     MV_REQUIRE(n >= 0 && QR > 0 && R > 0 && DR >= 0 && DR % 2 == 0, "latent_prepare: bad sizes n=%d QR=%d R=%d DR=%d", n, QR, R, DR);
     MV_REQUIRE(ld >= (long)QR + R + DR && ldq >= QR && page_size > 0 && bt_width > 0, "latent_prepare: row pitches too small");
     MV_REQUIRE(mv_valid_dtype(weight_dtype) && packed && wq && wkv && (table || DR == 0) && table_rows >= 0 && positions && token_seq
@@ -76,7 +83,7 @@ extern "C" int mv_latent_prepare(const void* packed, long ld, int n, int QR, int
     MV_DISPATCH_T(dtype, "latent_prepare",
                   hipLaunchKernelGGL(latent_prepare_kernel<T>, dim3(n), dim3(256), 0, stream, (const T*)packed, ld, QR, R, DR, a,
                                      b, eps, table, positions, token_seq, block_table, bt_width, page_size, (T*)cq, ldq,
-                                     (T*)pages));
+                                     (T*)pages, (T*)pages_t));
     return mv_check_launch("latent_prepare");
 }
 
@@ -584,3 +591,164 @@ extern "C" int mv_attention_latent_split(const float* q, long ldq, float* out, l
                        run, runs, out, ldo);
     return mv_check_launch("attention_latent_join");
 }
+
+
+#ifdef MV_WITH_BF16
+// ---------------------------------------------------------------------------------------
+// Attention for steps with prompt portions (bfloat16, MFMA). One wave per (row, group of 16 heads): the heads of a row
+// are the 16 rows of the first operand, since they all read the same key rows. Keys are walked 32 at a time from
+// position 0:   S = Q K^T (NQ products of 16 x 16 x 32 for each half of the block, key rows straight from the pages),
+// a running maximum and sum per head in float, P rounded to bfloat16 and turned from "a lane holds a key's column" to
+// "a lane holds a head's row" through the wave's own 1 KB of LDS,   O += P V with V from the pages that hold the
+// latents slot-contiguous (a lane's eight keys are eight neighbouring slots of one page: page_size % 8 == 0).
+// Keys behind the row's position are masked in S and zeroed in V (their slots may hold anything).
+// v_mfma_f32_16x16x32_bf16: lane l holds row l % 16 of the first operand (k = 8 (l / 16) .. + 7), column l % 16 of the
+// second, and column l % 16 of rows 4 (l / 16) .. + 3 of the result.
+// ---------------------------------------------------------------------------------------
+typedef __bf16 alm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float alm_f4 __attribute__((ext_vector_type(4)));
+union AlmFrag {
+    uint4 u;
+    alm_bf16x8 v;
+    uint16_t h[8];
+};
+
+__device__ __forceinline__ float alm_row16_max(float v) {
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float alm_row16_sum(float v) {
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+template <int NQ, int NR>
+__global__ void __launch_bounds__(256)
+attention_latent_mfma_kernel(const float* __restrict__ q, long ldq, float* __restrict__ out, long ldo, const bf16* __restrict__ pages,
+                             const bf16* __restrict__ pages_t, const int* __restrict__ block_table, int bt_width, int page_size,
+                             const int* __restrict__ positions, const int* __restrict__ token_seq, int n, int H, float scale) {
+    constexpr int DK = NQ * 32, R = NR * 16;
+    __shared__ __attribute__((aligned(16))) uint16_t pl[4][16][40];          // a wave's P: [head][key], rows 80 bytes apart
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const int tok = blockIdx.x * 4 + wave, h0 = blockIdx.y * 16;
+    if (tok >= n) return;
+    const int r = lane % 16, kq = lane / 16;
+    const int nh = min(16, H - h0);
+    const int seq = token_seq[tok];
+    if (seq < 0) {
+        for (int e = lane; e < nh * R; e += 64) out[(size_t)tok * ldo + (size_t)(h0 + e / R) * R + e % R] = 0.f;
+        return;
+    }
+    const int pos = positions[tok];
+    const int* bt = block_table + (size_t)seq * bt_width;
+    AlmFrag qf[NQ];
+#pragma unroll
+    for (int c = 0; c < NQ; ++c) {
+        if (r < nh) {
+            const float* src = q + (size_t)tok * ldq + (size_t)(h0 + r) * DK + 32 * c + 8 * kq;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qf[c].h[e] = f32_to_bf16_bits(src[e] * scale);
+        } else {
+            qf[c].u = uint4{0u, 0u, 0u, 0u};
+        }
+    }
+    float m[4], l[4];
+    alm_f4 acc[NR];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        m[i] = -INFINITY;
+        l[i] = 0.f;
+    }
+#pragma unroll
+    for (int t = 0; t < NR; ++t) acc[t] = alm_f4{0.f, 0.f, 0.f, 0.f};
+    for (int kb = 0; kb <= pos; kb += 32) {
+        alm_f4 s[2];
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            s[sub] = alm_f4{0.f, 0.f, 0.f, 0.f};
+            const int key = kb + 16 * sub + r;
+            const int kc = key <= pos ? key : pos;           // keys behind the row: some valid row, masked below
+            const bf16* krow = pages + ((size_t)bt[kc / page_size] * page_size + kc % page_size) * DK + 8 * kq;
+#pragma unroll
+            for (int c = 0; c < NQ; ++c) {
+                AlmFrag kf;
+                kf.u = *reinterpret_cast<const uint4*>(krow + 32 * c);
+                s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c].v, kf.v, s[sub], 0, 0, 0);
+            }
+        }
+        const bool ok0 = kb + r <= pos, ok1 = kb + 16 + r <= pos;
+        float corr[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float a = ok0 ? s[0][i] : -INFINITY, b = ok1 ? s[1][i] : -INFINITY;
+            const float m_new = fmaxf(m[i], alm_row16_max(fmaxf(a, b)));
+            const float p0 = ok0 ? expf(a - m_new) : 0.f, p1 = ok1 ? expf(b - m_new) : 0.f;
+            corr[i] = expf(m[i] - m_new);                    // first block: exp(-inf) = 0
+            l[i] = l[i] * corr[i] + alm_row16_sum(p0 + p1);
+            m[i] = m_new;
+            pl[wave][4 * kq + i][r] = f32_to_bf16_bits(p0);
+            pl[wave][4 * kq + i][16 + r] = f32_to_bf16_bits(p1);
+        }
+#pragma unroll
+        for (int t = 0; t < NR; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[t][i] *= corr[i];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        AlmFrag pf;
+        pf.u = *reinterpret_cast<const uint4*>(&pl[wave][r][8 * kq]);
+        const int key0 = kb + 8 * kq;                        // this lane's eight keys: one page's neighbouring slots
+        const int live = min(8, pos - key0 + 1);             // how many of them the row sees (<= 0: none)
+        // (every lane loads and multiplies, whatever it sees: a matrix instruction is the whole wave's. A lane that
+        // sees none of its keys reads the row's own page instead and zeroes all eight.)
+        const int keyc = live > 0 ? key0 : (pos / 8) * 8;
+        const bf16* vbase = pages_t + ((size_t)bt[keyc / page_size] * R + r) * page_size + keyc % page_size;
+#pragma unroll
+        for (int t = 0; t < NR; ++t) {
+            AlmFrag vf;
+            vf.u = *reinterpret_cast<const uint4*>(vbase + (size_t)16 * t * page_size);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (e >= live) vf.h[e] = 0;
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, vf.v, acc[t], 0, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int head = 4 * kq + i;
+        if (head < nh) {
+            const float inv = 1.f / l[i];
+#pragma unroll
+            for (int t = 0; t < NR; ++t) out[(size_t)tok * ldo + (size_t)(h0 + head) * R + 16 * t + r] = acc[t][i] * inv;
+        }
+    }
+}
+
+// returns 2 (nothing done) for sizes it does not serve: (R, DR) in (64, 32), (128, 32), (128, 64), (256, 64), pages
+// whose size is a multiple of 8
+extern "C" int mv_attention_latent_mfma(const float* q, long ldq, float* out, long ldo, const void* pages, const void* pages_t,
+                                        const int* block_table, int bt_width, int page_size, const int* positions,
+                                        const int* token_seq, int n, int H, int R, int DR, float scale, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && H > 0 && R > 0 && DR >= 0, "attention_latent_mfma: bad sizes n=%d H=%d R=%d DR=%d", n, H, R, DR);
+    const bool served = (R == 64 && DR == 32) || (R == 128 && DR == 32) || (R == 128 && DR == 64) || (R == 256 && DR == 64);
+    if (!served || page_size % 8 != 0 || !pages_t || ((uintptr_t)pages % 16) || ((uintptr_t)pages_t % 16)) return 2;
+    MV_REQUIRE(bt_width > 0 && ldq >= (long)H * (R + DR) && ldo >= (long)H * R, "attention_latent_mfma: pitches too small");
+    MV_REQUIRE(q && out && pages && block_table && positions && token_seq, "attention_latent_mfma: missing operand");
+    if (n == 0) return 0;
+    dim3 grid((n + 3) / 4, (H + 15) / 16);
+#define ALM_LAUNCH(NQ, NR)                                                                                                 \
+    hipLaunchKernelGGL((attention_latent_mfma_kernel<NQ, NR>), grid, dim3(256), 0, stream, q, ldq, out, ldo, (const bf16*)pages, \
+                       (const bf16*)pages_t, block_table, bt_width, page_size, positions, token_seq, n, H, scale)
+    if (R == 64) ALM_LAUNCH(3, 4);
+    else if (R == 128 && DR == 32) ALM_LAUNCH(5, 8);
+    else if (R == 128) ALM_LAUNCH(6, 8);
+    else ALM_LAUNCH(10, 16);
+#undef ALM_LAUNCH
+    return mv_check_launch("attention_latent_mfma");
+}
+#endif

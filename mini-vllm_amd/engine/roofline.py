@@ -63,6 +63,7 @@ KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
     "mv_latent_prepare": (r"\blatent_prepare_kernel", None, 1),
     "mv_head_linear": (r"\bhead_linear_kernel", None, 1),
     "mv_attention_latent": (r"\battention_latent_kernel", None, 1),
+    "mv_attention_latent_mfma": (r"\battention_latent_mfma_kernel", None, 1),
     "mv_attention_latent_split": (r"\battention_latent_split_kernel", r"\battention_latent_join_kernel", 2),
     "mv_moe_route": (r"\bmoe_route_kernel", None, 1),
     "mv_moe_swiglu_scale": (r"\bmoe_swiglu_scale_kernel", None, 1),

@@ -82,6 +82,9 @@ _SIGNATURES = {
 
 # entry points that only the bfloat16 library has
 _OPTIONAL_SIGNATURES = {
+    # q, ldq, out, ldo, pages, pages_t, block_table, bt_width, page_size, positions, token_seq, n, H, R, DR, scale, stream
+    "mv_attention_latent_mfma": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                                         c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "mv_moe_grouped_ints": (c_long, [c_int, c_int, c_int]),
     # x, ldx, n, hidden, w_gate_up, w_down, n_real, identity, F, ids, weights, top, dense, ld_dense, ints, act, out, y, ldy, stream
     "mv_moe_grouped": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int,
@@ -170,9 +173,9 @@ _OPTIONAL_SIGNATURES = {
     "mv_state_finish": (c_int, [c_void_p, c_void_p, c_void_p, c_long, c_long, c_void_p, c_int, c_int, c_int, c_int, c_float,
                                 c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_long, c_int, c_void_p]),
     # packed, ld, n, QR, R, DR, wq, wkv, weight_dtype, eps, table, table_rows, positions, token_seq, block_table, bt_width,
-    # page_size, cq, ldq, pages, dtype, stream
+    # page_size, cq, ldq, pages, pages_t, dtype, stream
     "mv_latent_prepare": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
-                                  c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_int,
+                                  c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_int,
                                   c_void_p]),
     # x, ldx, ldx_head, w, weight_dtype, n, H, IN, OUT, y, ldy, ldy_head, tail, table, positions, gate, ldg, token_seq, mode,
     # dtype, stream

@@ -726,10 +726,11 @@ class Ops:
     def latent_prepare(self, packed: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, q_norm: torch.Tensor,
                        kv_norm: torch.Tensor, eps: float, table: Optional[torch.Tensor], positions: torch.Tensor,
                        token_seq: torch.Tensor, block_table: torch.Tensor, page_size: int, q_latent: torch.Tensor,
-                       pages: torch.Tensor) -> None:
+                       pages: torch.Tensor, pages_t: Optional[torch.Tensor] = None) -> None:
         """From rows [dq (q_rank) | dkv (kv_rank + rot_dim) | ...]: q_latent = rmsnorm(dq) * q_norm; the row's cache
         entry [rmsnorm(dkv[:kv_rank]) * kv_norm | rot(dkv[kv_rank:])] goes to pages [pages, page_size, kv_rank + rot_dim]
-        at the row's position (``table``: float32 [positions, rot_dim] = cat(cos, sin), pairs i, i + rot_dim/2)."""
+        at the row's position (``table``: float32 [positions, rot_dim] = cat(cos, sin), pairs i, i + rot_dim/2).
+        ``pages_t`` [pages, kv_rank, page_size], when given, gets the latent once more, a page's slots side by side."""
         self._act(packed, "latent rows"); self._act(q_latent, "query latent"); self._act(pages, "latent pages")
         n = packed.shape[0]
         if packed.dim() != 2 or packed.stride(1) != 1 or packed.shape[1] < q_rank + kv_rank + rot_dim:
@@ -742,6 +743,10 @@ class Ops:
             _dev(t, name)
             if t.numel() != size or not t.is_contiguous() or t.dtype != q_norm.dtype:
                 raise KernelLibraryError(f"latent_prepare: the {name} weight must hold {size} numbers")
+        if pages_t is not None:
+            self._act(pages_t, "slot-contiguous latent pages")
+            if tuple(pages_t.shape) != (pages.shape[0], kv_rank, page_size) or not pages_t.is_contiguous():
+                raise KernelLibraryError(f"latent_prepare: the slot-contiguous pages must be [{pages.shape[0]}, {kv_rank}, {page_size}]")
         rows = 0
         if rot_dim:
             _dev(table, "rotary table")
@@ -757,7 +762,7 @@ class Ops:
                       rot_dim, q_norm.data_ptr(), kv_norm.data_ptr(), _weight_code(q_norm, "latent norm"), float(eps),
                       _ptr(table), rows, positions.data_ptr(), token_seq.data_ptr(), block_table.data_ptr(),
                       block_table.shape[1], page_size, q_latent.data_ptr(), q_latent.stride(0) if n > 1 else q_rank,
-                      pages.data_ptr(), self.code, self._stream())
+                      pages.data_ptr(), _ptr(pages_t), self.code, self._stream())
 
     def head_linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, token_seq: torch.Tensor, tail: int = 0,
                     table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
@@ -801,10 +806,12 @@ class Ops:
 
     def attention_latent(self, q: torch.Tensor, out: torch.Tensor, pages: torch.Tensor, block_table: torch.Tensor,
                          page_size: int, positions: torch.Tensor, token_seq: torch.Tensor, heads: int, kv_rank: int,
-                         rot_dim: int, scale: float, plan=None) -> None:
+                         rot_dim: int, scale: float, plan=None, pages_t: Optional[torch.Tensor] = None) -> None:
         """Causal softmax attention of q float32 [n, heads, kv_rank + rot_dim] over the cached rows [latent | rotated
         key part] of each row's request (pages [pages, page_size, kv_rank + rot_dim]); out float32 [n, heads, kv_rank] is
-        the weighted sum of the latents."""
+        the weighted sum of the latents. Steps of single tokens take the kernel that deals a row's keys out over workgroups;
+        in bfloat16 other steps take the MFMA kernel where it serves the sizes (it reads the values from ``pages_t``
+        [pages, kv_rank, page_size], the latents with a page's slots side by side); everything else the general kernel."""
         _dev(q, "latent queries"); _dev(out, "latent attention output"); self._act(pages, "latent pages")
         n, dk = q.shape[0], kv_rank + rot_dim
         if q.dtype != torch.float32 or tuple(q.shape) != (n, heads, dk) or not q.is_contiguous():
@@ -823,6 +830,17 @@ class Ops:
                 q, out, pages, block_table, page_size, positions, token_seq, n, heads, kv_rank, rot_dim, scale,
                 plan.max_context_len, kv_tokens):
             return
+        if pages_t is not None and self.use_fast_kernels and self.lib.has("mv_attention_latent_mfma") \
+                and not (plan is not None and plan.decode_only):
+            self._act(pages_t, "slot-contiguous latent pages")
+            if tuple(pages_t.shape) != (pages.shape[0], kv_rank, page_size) or not pages_t.is_contiguous():
+                raise KernelLibraryError(f"attention_latent: the slot-contiguous pages must be [{pages.shape[0]}, {kv_rank}, {page_size}]")
+            if self.lib.offer("mv_attention_latent_mfma", q.data_ptr(), heads * dk, out.data_ptr(), heads * kv_rank, pages.data_ptr(),
+                              pages_t.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size, positions.data_ptr(),
+                              token_seq.data_ptr(), n, heads, kv_rank, rot_dim, float(scale), self._stream()):
+                self._note("mv_attention_latent_mfma", self._size(q, out) + kv_tokens * (dk + kv_rank) * pages.element_size(),
+                           2 * pairs * heads * (dk + kv_rank))
+                return
         self._note("mv_attention_latent", self._size(q, out) + kv_tokens * dk * pages.element_size(),
                    2 * pairs * heads * (dk + kv_rank))
         self.lib.call("mv_attention_latent", q.data_ptr(), heads * dk, out.data_ptr(), heads * kv_rank, pages.data_ptr(),

@@ -12,8 +12,8 @@ Head h's key is [W_uk,h c | k_rot] and its value W_uv,h c; the score of query i 
 outputs are concatenated, multiplied by sigmoid(W_g h) when ``output_gate`` is set, and projected
 by W_o.
 
-Only [c | k_rot] is cached, one row of ``kv_rank + rot_dim`` numbers per token
-(``LatentNeed``). Keys and values are never expanded: the query is carried into the latent's space
+Only [c | k_rot] is cached, one row of ``kv_rank + rot_dim`` numbers per token, and c once more in
+the slot-contiguous layout that the MFMA kernel's second product reads (``LatentNeed``). Keys and values are never expanded: the query is carried into the latent's space
 (W_uk,h^T q_plain), attention runs on the cached rows with the latent as the value, and W_uv,h is
 applied to the weighted sum of latents. Norms, rotation, scores, weights and sums are float32.
 """
@@ -29,12 +29,18 @@ from .base import CacheNeed, KeepAll, Mixer, PartSpec, Retention, Runtime, Tenso
 
 @dataclass(frozen=True)
 class LatentNeed(CacheNeed):
-    """One row per token: the latent and the rotated key part side by side."""
+    """One row per token: the latent and the rotated key part side by side (``latent``). With ``latent_dim`` the latent
+    is kept once more with a page's slots side by side (``latent_t`` [latent_dim, slot]): the second product of an MFMA
+    attention kernel reads eight neighbouring keys of one channel in one load from there."""
     retention: Retention
     width: int
+    latent_dim: int = 0
 
     def page_shapes(self, page_size: int) -> Dict[str, Tuple[int, ...]]:
-        return {"latent": (page_size, self.width)}
+        shapes = {"latent": (page_size, self.width)}
+        if self.latent_dim:
+            shapes["latent_t"] = (self.latent_dim, page_size)
+        return shapes
 
 
 @dataclass(frozen=True)
@@ -71,7 +77,7 @@ class LatentAttention(Mixer):
 
     @classmethod
     def cache_need(cls, spec: LatentAttentionSpec) -> Optional[CacheNeed]:
-        return LatentNeed(retention=KeepAll(), width=spec.kv_rank + spec.rot_dim)
+        return LatentNeed(retention=KeepAll(), width=spec.kv_rank + spec.rot_dim, latent_dim=spec.kv_rank)
 
     def __init__(self, spec: LatentAttentionSpec, tensors: Dict[str, torch.Tensor], rt: Runtime, position: Optional[object] = None):
         if min(spec.num_heads, spec.plain_dim, spec.value_dim, spec.q_rank, spec.kv_rank) < 1 or spec.rot_dim < 0 or spec.rot_dim % 2:
@@ -109,10 +115,10 @@ class LatentAttention(Mixer):
         packed = ws.get("latent.packed", (n, self.width), rt.dtype)
         ops.gemm(x, self.w_packed, packed)
         kv = ctx.kv(call)
-        pages = kv.pages["latent"]
+        pages, pages_t = kv.pages["latent"], kv.pages.get("latent_t")
         cq = ws.get("latent.cq", (n, spec.q_rank), rt.dtype)
         ops.latent_prepare(packed, spec.q_rank, R, dr, self.q_norm, self.kv_norm, spec.norm_eps, self.table, ctx.positions,
-                           ctx.token_seq, kv.block_table, kv.page_size, cq, pages)
+                           ctx.token_seq, kv.block_table, kv.page_size, cq, pages, pages_t)
         q = ws.get("latent.q", (n, H * (spec.plain_dim + dr)), rt.dtype)
         ops.gemm(cq, self.w_uq, q)
         qa = ws.get("latent.qa", (n, H, R + dr), torch.float32)
@@ -120,7 +126,7 @@ class LatentAttention(Mixer):
                         positions=ctx.positions)
         mixed = ws.get("latent.mixed", (n, H, R), torch.float32)
         ops.attention_latent(qa, mixed, pages, kv.block_table, kv.page_size, ctx.positions, ctx.token_seq, H, R, dr,
-                             spec.scale, plan=ctx.attention_plan)
+                             spec.scale, plan=ctx.attention_plan, pages_t=pages_t)
         heads = ws.get("latent.heads", (n, H * spec.value_dim), rt.dtype)
         gate = packed[:, self.gate_offset:self.gate_offset + H * spec.value_dim] if spec.output_gate else None
         ops.head_linear(mixed, self.w_uv, heads, ctx.token_seq, gate=gate)

@@ -72,8 +72,8 @@ def test_plan_parts_and_memory():
     assert states["state"] == ((4, 24, 16), torch.float32) and states["conv"][0] == (3, 2 * 2 * 16 + 4 * 24)
     assert MIXERS.get(ml.kind).state_shapes(ml) == {"state": ((2, 21, 16), torch.float32), "max": ((2,), torch.float32)}
     need = MIXERS.get(la.kind).cache_need(la)
-    assert need.page_shapes(8) == {"latent": (8, 32 + 8)} and isinstance(need.retention, KeepAll)
-    assert need.bytes_per_token(torch.bfloat16) == 80 and MIXERS.get(d.kind).cache_need(d) is None
+    assert need.page_shapes(8) == {"latent": (8, 32 + 8), "latent_t": (32, 8)} and isinstance(need.retention, KeepAll)
+    assert need.bytes_per_token(torch.bfloat16) == 80 + 64 and MIXERS.get(d.kind).cache_need(d) is None
     r = plan.layers[0].ffn
     assert (r.num_experts, r.identity_experts, r.top, r.groups, r.keep_groups, r.router_outputs) == (8, 2, 3, 5, 3, 10)
     # the two attention layers keep everything: one cache group

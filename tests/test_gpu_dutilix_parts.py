@@ -556,6 +556,61 @@ def test_latent_attention_single_token_kernel(dtype, H, R, dr):
     close(fast[:-1], slow[:-1].double(), 3e-5, "against the general kernel")
 
 
+@pytest.mark.parametrize("H, R, dr", [(16, 256, 64), (5, 64, 32), (20, 128, 32), (8, 128, 64)])
+@pytest.mark.parametrize("page_size", [16, 8])
+def test_latent_attention_mfma_kernel(H, R, dr, page_size):
+    """bfloat16 steps with prompt portions take an MFMA kernel (a row's 16 heads are the rows of its first operand, the
+    values come from the slot-contiguous pages): a prompt of 100 tokens, a portion that starts in the middle of a block of
+    32 keys, single rows at positions 0, 31, 32, 33 and 700, a padding row; NaN in every slot nobody wrote. Against the
+    softmax written out on the stored rows."""
+    from minivllm_amd.engine.step import AttentionPlan
+    dtype = torch.bfloat16
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(H + R)
+    ctx = [100, 77, 1, 32, 33, 34, 701]                    # contexts of the seven requests after the step
+    qlens = [100, 20, 1, 1, 1, 1, 1]
+    n_pages = sum(-(-c // page_size) for c in ctx) + 3
+    pages = torch.full((n_pages, page_size, R + dr), float("nan"), dtype=dtype, device=DEV)
+    pages_t = torch.full((n_pages, R, page_size), float("nan"), dtype=dtype, device=DEV)
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    width = -(-max(ctx) // page_size)
+    bt = torch.full((len(ctx), width), -1, dtype=torch.int32)
+    rows, used = [], 0
+    for s_, c in enumerate(ctx):
+        need = -(-c // page_size)
+        bt[s_, :need] = torch.tensor(perm[used:used + need], dtype=torch.int32)
+        used += need
+        data = torch.randn(c, R + dr, generator=g).to(dtype)
+        rows.append(data)
+        for p_ in range(c):
+            pages[bt[s_, p_ // page_size], p_ % page_size] = data[p_].to(DEV)
+            pages_t[bt[s_, p_ // page_size], :, p_ % page_size] = data[p_, :R].to(DEV)
+    pos, tsq = [], []
+    for s_, (c, ql) in enumerate(zip(ctx, qlens)):
+        pos += list(range(c - ql, c)); tsq += [s_] * ql
+    pos.append(0); tsq.append(-1)
+    n = len(pos)
+    qa = (1.2 * torch.randn(n, H, R + dr, generator=g)).to(DEV)
+    plan = AttentionPlan(decode_only=False, max_q_len=100, max_context_len=1024, n_seqs=len(ctx))
+    got = torch.full((n, H, R), float("nan"), device=DEV)
+    ops.ledger = []
+    ops.attention_latent(qa, got, pages, bt.to(DEV), page_size, i32(pos), i32(tsq), H, R, dr, 0.15, plan=plan, pages_t=pages_t)
+    torch.cuda.synchronize()
+    assert [e[0] for e in ops.ledger] == ["mv_attention_latent_mfma"]
+    ops.ledger = None
+    bad = (~torch.isfinite(got)).nonzero()
+    assert bad.numel() == 0, f"non-finite outputs at (row, head, channel) {bad[:8].tolist()} ... of rows at positions {sorted({pos[i] for i in bad[:, 0].tolist()})[:12]}"
+    assert (got[-1] == 0).all()
+    worst = 0.0
+    for t in range(n - 1):
+        look = rows[tsq[t]][:pos[t] + 1].double()
+        for h in range(H):
+            w = torch.softmax(look @ qa[t, h].double().cpu() * 0.15, 0)
+            want = w @ look[:, :R]
+            worst = max(worst, float((got[t, h].double().cpu() - want).abs().max() / want.abs().max()))
+    assert worst < 2e-2, worst
+
+
 # ---------------------------------------------------------------------------------------
 # router and experts
 # ---------------------------------------------------------------------------------------
