@@ -752,3 +752,111 @@ extern "C" int mv_attention_latent_mfma(const float* q, long ldq, float* out, lo
     return mv_check_launch("attention_latent_mfma");
 }
 #endif
+
+#ifdef MV_WITH_BF16
+// ---------------------------------------------------------------------------------------
+// The per-head maps for steps of many rows (bfloat16, MFMA): y[t][h] = W_h x[t][h] with w [H][OUT][IN], the inputs of an
+// output row side by side (the other layout than head_linear's). A workgroup takes 64 rows, one head and 128 output
+// columns; each of its four waves 16 rows x 128 columns (v_mfma_f32_16x16x32_bf16, operands straight from memory; lane
+// l holds row l % 16 of x, column l % 16 of the weight, 8 inputs from 8 (l / 16)). IN must be a multiple of 32.
+//   mode 0   x bfloat16 [n][H][IN + tail] -> y float [n][H][OUT + tail], the tail rotated by the row's position
+//   mode 1   x float [n][H][IN] (rounded to bfloat16 as it is read) -> y bfloat16 [n][H * OUT], times sigmoid(gate)
+// ---------------------------------------------------------------------------------------
+template <int MODE>
+__global__ void __launch_bounds__(256)
+head_linear_mfma_kernel(const void* __restrict__ xv, long ldx, int ldx_head, const bf16* __restrict__ w, int IN, int OUT,
+                        void* __restrict__ yv, long ldy, int ldy_head, int tail, const float* __restrict__ table,
+                        const int* __restrict__ positions, const bf16* __restrict__ gate, long ldg,
+                        const int* __restrict__ token_seq, int n) {
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int t0 = blockIdx.x * 64 + 16 * wave, head = blockIdx.y, n0 = blockIdx.z * 128;
+    if (t0 >= n) return;                                     // (the whole wave: its 16 rows are past the end)
+    const int r = lane % 16, kq = lane / 16;
+    const int trow = min(t0 + r, n - 1);                     // rows past the end: the last row; never stored
+    const bf16* wrow[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        const int col = min(n0 + 16 * s + r, OUT - 1);       // columns past the end: the last column; never stored
+        wrow[s] = w + ((size_t)head * OUT + col) * IN + 8 * kq;
+    }
+    alm_f4 acc[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) acc[s] = alm_f4{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < IN; k0 += 32) {
+        AlmFrag fa;
+        if (MODE == 0) {
+            const bf16* x = (const bf16*)xv + (size_t)trow * ldx + (size_t)head * ldx_head + k0 + 8 * kq;
+            if ((((uintptr_t)x) & 15) == 0) {
+                fa.u = *reinterpret_cast<const uint4*>(x);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) fa.h[e] = x[e].bits;
+            }
+        } else {
+            const float* x = (const float*)xv + (size_t)trow * ldx + (size_t)head * ldx_head + k0 + 8 * kq;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) fa.h[e] = f32_to_bf16_bits(x[e]);
+        }
+        AlmFrag fb[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) fb[s].u = *reinterpret_cast<const uint4*>(wrow[s] + k0);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa.v, fb[s].v, acc[s], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int t = t0 + 4 * kq + i;
+        if (t >= n) continue;
+        const bool pad = token_seq[t] < 0;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int col = n0 + 16 * s + r;
+            if (col >= OUT) continue;
+            float v = pad ? 0.f : acc[s][i];
+            if (MODE == 0) {
+                ((float*)yv)[(size_t)t * ldy + (size_t)head * ldy_head + col] = v;
+            } else {
+                if (gate && !pad) v *= 1.f / (1.f + expf(-to_f(gate[(size_t)t * ldg + (size_t)head * OUT + col])));
+                ((bf16*)yv)[(size_t)t * ldy + (size_t)head * ldy_head + col] = from_f<bf16>(v);
+            }
+        }
+    }
+    if (MODE == 0 && blockIdx.z == 0 && tail > 0) {
+        const int half = tail / 2;
+        const int rows = min(16, n - t0);
+        for (int e = lane; e < rows * half; e += 64) {
+            const int t = t0 + e / half, i = e % half;
+            const bf16* src = (const bf16*)xv + (size_t)t * ldx + (size_t)head * ldx_head + IN;
+            float* dst = (float*)yv + (size_t)t * ldy + (size_t)head * ldy_head + OUT;
+            if (token_seq[t] < 0) {
+                dst[i] = 0.f;
+                dst[half + i] = 0.f;
+                continue;
+            }
+            const float* cs = table + (size_t)positions[t] * tail;
+            const float a = to_f(src[i]), b = to_f(src[half + i]);
+            dst[i] = a * cs[i] - b * cs[half + i];
+            dst[half + i] = b * cs[i] + a * cs[half + i];
+        }
+    }
+}
+
+// returns 2 (nothing done) for sizes it does not serve
+extern "C" int mv_head_linear_mfma(const void* x, long ldx, int ldx_head, const void* w, int n, int H, int IN, int OUT, void* y,
+                                   long ldy, int ldy_head, int tail, const float* table, const int* positions, const void* gate,
+                                   long ldg, const int* token_seq, int mode, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && H > 0 && IN > 0 && OUT > 0 && tail >= 0 && tail % 2 == 0, "head_linear_mfma: bad sizes");
+    if (IN % 32 != 0 || ((uintptr_t)w % 16) != 0 || (mode == 1 && (ldx % 4 || ldx_head % 4))) return 2;
+    MV_REQUIRE(ldx_head >= IN + tail && ldy_head >= OUT + (mode == 0 ? tail : 0) && x && w && y && token_seq && H <= 65535
+               && (tail == 0 || (table && positions)) && (mode == 0 ? !gate : tail == 0), "head_linear_mfma: operands do not fit");
+    if (n == 0) return 0;
+    dim3 grid((n + 63) / 64, H, (OUT + 127) / 128);
+    if (mode == 0)
+        hipLaunchKernelGGL(head_linear_mfma_kernel<0>, grid, dim3(256), 0, stream, x, ldx, ldx_head, (const bf16*)w, IN, OUT, y, ldy,
+                           ldy_head, tail, table, positions, (const bf16*)nullptr, 0L, token_seq, n);
+    else
+        hipLaunchKernelGGL(head_linear_mfma_kernel<1>, grid, dim3(256), 0, stream, x, ldx, ldx_head, (const bf16*)w, IN, OUT, y, ldy,
+                           ldy_head, 0, table, positions, (const bf16*)gate, ldg, token_seq, n);
+    return mv_check_launch("head_linear_mfma");
+}
+#endif

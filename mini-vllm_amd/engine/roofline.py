@@ -62,6 +62,7 @@ KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
     "mv_state_step": (r"\bstate_step_kernel", r"\bconv_state_kernel", 2),
     "mv_latent_prepare": (r"\blatent_prepare_kernel", None, 1),
     "mv_head_linear": (r"\bhead_linear_kernel", None, 1),
+    "mv_head_linear_mfma": (r"\bhead_linear_mfma_kernel", None, 1),
     "mv_attention_latent": (r"\battention_latent_kernel", None, 1),
     "mv_attention_latent_mfma": (r"\battention_latent_mfma_kernel", None, 1),
     "mv_attention_latent_split": (r"\battention_latent_split_kernel", r"\battention_latent_join_kernel", 2),

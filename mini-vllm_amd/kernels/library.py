@@ -82,6 +82,9 @@ _SIGNATURES = {
 
 # entry points that only the bfloat16 library has
 _OPTIONAL_SIGNATURES = {
+    # x, ldx, ldx_head, w, n, H, IN, OUT, y, ldy, ldy_head, tail, table, positions, gate, ldg, token_seq, mode, stream
+    "mv_head_linear_mfma": (c_int, [c_void_p, c_long, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_long, c_int, c_int,
+                                    c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p]),
     # q, ldq, out, ldo, pages, pages_t, block_table, bt_width, page_size, positions, token_seq, n, H, R, DR, scale, stream
     "mv_attention_latent_mfma": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                          c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p]),

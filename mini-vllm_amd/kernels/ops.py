@@ -766,11 +766,13 @@ class Ops:
 
     def head_linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, token_seq: torch.Tensor, tail: int = 0,
                     table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
-                    gate: Optional[torch.Tensor] = None) -> None:
+                    gate: Optional[torch.Tensor] = None, w_rows: Optional[torch.Tensor] = None) -> None:
         """Per head h: out[t, h, :OUT] = x[t, h, :IN] @ w[h] with w [heads, IN, OUT]. x [n, heads, IN + tail] in the
         activation type gives out float32 [n, heads, OUT + tail], the ``tail`` last inputs copied behind the outputs
         and rotated by the row's position (``table`` as for ``latent_prepare``); x float32 [n, heads, IN] gives out
-        [n, heads * OUT] in the activation type, multiplied by sigmoid(gate [n, heads * OUT]) when a gate is given."""
+        [n, heads * OUT] in the activation type, multiplied by sigmoid(gate [n, heads * OUT]) when a gate is given.
+        ``w_rows`` is the same weight as [heads, OUT, IN]: in bfloat16, steps of more than 64 rows whose IN is a multiple
+        of 32 take the MFMA kernel, which reads that layout (and rounds float32 inputs to bfloat16 as it reads them)."""
         _dev(x, "head_linear input"); _dev(w, "head_linear weight"); _dev(out, "head_linear output")
         if w.dim() != 3 or not w.is_contiguous() or x.dim() != 3 or x.stride(2) != 1 or x.stride(1) != x.shape[2]:
             raise KernelLibraryError("head_linear: x [n, heads, width] and a contiguous w [heads, IN, OUT] are needed")
@@ -798,6 +800,16 @@ class Ops:
                     raise KernelLibraryError("head_linear: the gate must be [n, heads * OUT]")
         else:
             raise KernelLibraryError(f"head_linear: {x.dtype} -> {out.dtype} with these options is not served")
+        if w_rows is not None and n > 64 and self.use_fast_kernels and w_rows.dtype == torch.bfloat16 \
+                and self.lib.has("mv_head_linear_mfma"):
+            _dev(w_rows, "head_linear weight")
+            if tuple(w_rows.shape) != (H, OUT, IN) or not w_rows.is_contiguous():
+                raise KernelLibraryError(f"head_linear: the row layout of the weight must be [{H}, {OUT}, {IN}]")
+            if self.lib.offer("mv_head_linear_mfma", x.data_ptr(), x.stride(0), x.shape[2], w_rows.data_ptr(), n, H, IN, OUT,
+                              out.data_ptr(), ldy, ldy_head, tail, _ptr(table), _ptr(positions), _ptr(gate),
+                              gate.stride(0) if gate is not None else 0, token_seq.data_ptr(), mode, self._stream()):
+                self._note("mv_head_linear_mfma", self._size(x, w, out), 2 * n * H * IN * OUT)
+                return
         self._note("mv_head_linear", self._size(x, w, out), 2 * n * H * IN * OUT)
         self.lib.call("mv_head_linear", x.data_ptr(), x.stride(0) if n > 1 else H * x.shape[2], x.shape[2], w.data_ptr(),
                       _weight_code(w, "head_linear weight"), n, H, IN, OUT, out.data_ptr(), ldy, ldy_head, tail, _ptr(table),

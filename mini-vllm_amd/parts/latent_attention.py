@@ -107,6 +107,9 @@ class LatentAttention(Mixer):
         # [heads, inputs, outputs]: the stored W_uk is that already; W_uv is stored [heads * value_dim, kv_rank]
         self.w_uk = tensors["uk"].view(spec.num_heads, spec.plain_dim, spec.kv_rank).contiguous()
         self.w_uv = tensors["uv"].view(spec.num_heads, spec.value_dim, spec.kv_rank).transpose(1, 2).contiguous()
+        # ... and both as [heads, outputs, inputs], which the MFMA kernel of steps with many rows reads
+        self.w_uk_rows = self.w_uk.transpose(1, 2).contiguous()
+        self.w_uv_rows = tensors["uv"].view(spec.num_heads, spec.value_dim, spec.kv_rank).contiguous()
         self.w_o = tensors["o"]
 
     def forward(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
@@ -123,12 +126,12 @@ class LatentAttention(Mixer):
         ops.gemm(cq, self.w_uq, q)
         qa = ws.get("latent.qa", (n, H, R + dr), torch.float32)
         ops.head_linear(q.view(n, H, spec.plain_dim + dr), self.w_uk, qa, ctx.token_seq, tail=dr, table=self.table,
-                        positions=ctx.positions)
+                        positions=ctx.positions, w_rows=self.w_uk_rows)
         mixed = ws.get("latent.mixed", (n, H, R), torch.float32)
         ops.attention_latent(qa, mixed, pages, kv.block_table, kv.page_size, ctx.positions, ctx.token_seq, H, R, dr,
                              spec.scale, plan=ctx.attention_plan, pages_t=pages_t)
         heads = ws.get("latent.heads", (n, H * spec.value_dim), rt.dtype)
         gate = packed[:, self.gate_offset:self.gate_offset + H * spec.value_dim] if spec.output_gate else None
-        ops.head_linear(mixed, self.w_uv, heads, ctx.token_seq, gate=gate)
+        ops.head_linear(mixed, self.w_uv, heads, ctx.token_seq, gate=gate, w_rows=self.w_uv_rows)
         y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
         return ops.gemm(heads, self.w_o, y, defer_sum=True) or y

@@ -611,6 +611,49 @@ def test_latent_attention_mfma_kernel(H, R, dr, page_size):
     assert worst < 2e-2, worst
 
 
+@pytest.mark.parametrize("H, IN, OUT, tail, n", [(16, 128, 256, 64, 300), (3, 32, 40, 8, 70), (5, 64, 128, 0, 130), (2, 96, 17, 4, 65)])
+def test_per_head_maps_mfma_against_the_general_kernel(H, IN, OUT, tail, n):
+    """bfloat16 steps of more than 64 rows take an MFMA kernel for the per-head maps: both directions (queries into latent
+    space with the rotated tail; weighted latents into values with the gate), padding rows, against the general kernel
+    and against the sums written out."""
+    dtype = torch.bfloat16
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(IN + OUT)
+    w = (torch.randn(H, IN, OUT, generator=g) / IN ** 0.5).to(dtype).to(DEV)
+    w_rows = w.transpose(1, 2).contiguous()
+    tsq = i32([0] * (n - 2) + [-1, -1])
+    pos = i32(list(range(n - 2)) + [0, 0])
+    table = ops.rope_table((1.0 / (10000.0 ** (torch.arange(0, tail, 2, dtype=torch.float) / tail))).to(DEV), 1024) if tail else None
+    # queries -> latent space
+    x = torch.randn(n, H, IN + tail, generator=g).to(dtype).to(DEV)
+    outs = []
+    for rows in (w_rows, None):
+        out = torch.full((n, H, OUT + tail), float("nan"), device=DEV)
+        ops.ledger = []
+        ops.head_linear(x, w, out, tsq, tail=tail, table=table, positions=pos, w_rows=rows)
+        torch.cuda.synchronize()
+        assert [e[0] for e in ops.ledger] == ["mv_head_linear_mfma" if rows is not None else "mv_head_linear"]
+        ops.ledger = None
+        outs.append(out)
+    want = torch.einsum("thi,hio->tho", x[..., :IN].double(), w.double())
+    close(outs[0][:-2, :, :OUT], want[:-2], 1e-5, "queries into latent space")
+    close(outs[0][:-2], outs[1][:-2].double(), 1e-5, "against the general kernel, tail included")
+    assert (outs[0][-2:] == 0).all()
+    # weighted latents -> values, gated
+    lat = torch.randn(n, H, IN, generator=g).to(DEV)
+    gate = torch.randn(n, H * OUT, generator=g).to(dtype).to(DEV)
+    outs = []
+    for rows in (w_rows, None):
+        out = torch.full((n, H * OUT), float("nan"), dtype=dtype, device=DEV)
+        ops.head_linear(lat, w, out, tsq, gate=gate, w_rows=rows)
+        torch.cuda.synchronize()
+        outs.append(out)
+    want = (torch.einsum("thi,hio->tho", lat.double(), w.double()).reshape(n, H * OUT) * torch.sigmoid(gate.double()))
+    close(outs[0][:-2], want[:-2], 1.2e-2, "weighted latents into values")
+    close(outs[0][:-2], outs[1][:-2].double(), 1.2e-2, "against the general kernel")
+    assert (outs[0][-2:] == 0).all()
+
+
 # ---------------------------------------------------------------------------------------
 # router and experts
 # ---------------------------------------------------------------------------------------
